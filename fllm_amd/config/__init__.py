@@ -1,6 +1,7 @@
 from .spec import ConfigError, LayerSpec, ModelSpec, PartSpec, RunEntry, default_run_order
 from .files import read_config_json
 from .llama import LlamaConfig, RopeScaling
+from .menitar import MenitarConfig
 
 __all__ = ["ConfigError", "LayerSpec", "ModelSpec", "PartSpec", "RunEntry", "default_run_order",
-           "LlamaConfig", "RopeScaling", "read_config_json"]
+           "LlamaConfig", "MenitarConfig", "RopeScaling", "read_config_json"]

@@ -58,10 +58,13 @@ class LayerSpec:
 class RunEntry:
     """One entry of the run order.  `layer` indexes `ModelSpec.layers` (a layer may be named by
     several entries: its weights run twice, each run with a cache of its own).  `reads_cache_of`
-    names an earlier entry whose cache this entry reads instead of writing one."""
+    names an earlier entry whose cache this entry reads instead of writing one.  `before`: a part of role
+    `stream` that changes the residual stream before the entry's layer runs (what a pass of looped layers adds to its
+    input); it may hold weights."""
 
     layer: int
     reads_cache_of: Optional[int] = None
+    before: Optional[PartSpec] = None
 
 
 @dataclass(frozen=True)

@@ -249,6 +249,41 @@ int fllm_logprobs_processed(const float *logits, int rows, int vocab, const int3
 int fllm_sample(const float *logits, float *work, const struct FllmSampleRow *params, int32_t *out, int rows, int vocab,
                 int kinds, hipStream_t stream);
 
+// ---- parts of other layer designs -------------------------------------------------------------------------------
+// Two RMSNorms of the same float32 rows in one pass: out1 = x * rsqrt(mean(x^2) + eps1) * w1, out2 likewise with w2
+// and eps2 (w2 and out2 null: one norm).  For blocks whose branches read the same residual stream.
+int fllm_rmsnorm_pair(const float *x, const float *w1, const float *w2, void *out1, void *out2, int rows, int width,
+                      float eps1, float eps2, int out_dtype, hipStream_t stream);
+// out[r, j] = g * sigmoid(alpha * g) * (u + up_offset), g = min(gu[r, j], limit), u = clamp(gu[r, I + j], -limit, limit)
+// (limit <= 0: nothing is clamped)
+int fllm_glu_clamped(const void *gate_up, void *out, int rows, int inter, float limit, float alpha, float up_offset, int dtype,
+                     hipStream_t stream);
+// x[i] *= scale
+int fllm_scale_f32(float *x, size_t total, float scale, hipStream_t stream);
+// x[r, :] = (x[r, :] + scale * table[ids[r], :]) + vec[:]; table (with ids) or vec may be null
+int fllm_stream_add(float *x, const int32_t *ids, const void *table, int table_dtype, int vocab, float scale, const float *vec,
+                    int rows, int width, hipStream_t stream);
+
+// Rows of a joint q/k/v product (row stride ld; queries first, then keys, then values): RMSNorm over the whole query
+// projection with q_weight [heads * k_dim] and over the whole key projection with k_weight [kv_heads * k_dim], rotary on
+// the first rope_dims lanes of every query and key head (lane i with lane i + rope_dims / 2; float32 tables [positions,
+// rope_dims / 2]); queries to q_out [rows, heads * k_dim], keys and values into the pages of the row's request.
+// K pages: [page][kv_head][k_dim / key_chunk][token][key_chunk]; V pages: [page][kv_head][v_dim][token].
+int fllm_qk_norm_rope_store(const void *qkv, int ld, const float *q_weight, const float *k_weight, float eps, void *q_out,
+                            const int32_t *row_pos, const int32_t *row_seg, const int32_t *tables, int table_stride,
+                            const float *cos_table, const float *sin_table, int table_positions, void *k_pages, void *v_pages,
+                            int rows, int heads, int kv_heads, int k_dim, int v_dim, int rope_dims, int page_size, int key_chunk,
+                            int dtype, int store_kv, hipStream_t stream);
+// Attention whose scores are mixed across heads before the softmax: score[h] = sum_g talk[h, g] * (q_g . k * scale *
+// temp[g]) over the keys lo .. pos of the row's request, lo = pos - pos % chunk (chunk 0: lo = 0); out[h] = gate *
+// softmax(score[h]) v, gate = sigmoid(gate[row * gate_stride + h]) (gate null: 1).  q: [rows, heads * k_dim]; out:
+// [rows, heads * v_dim]; talk float32 [heads, heads], temp float32 [heads].  Rows, segments and tables as fllm_attention.
+int fllm_talking_attention(const void *q, const void *gate, int gate_stride, const void *k_pages, const void *v_pages,
+                           const int32_t *tables, int table_stride, const int32_t *row_pos, const int32_t *row_seg,
+                           const int32_t *seg_start, int num_segs, const float *talk, const float *temp, void *out, int rows,
+                           int heads, int kv_heads, int k_dim, int v_dim, int page_size, float scale, int chunk, int key_chunk,
+                           int dtype, int max_context, hipStream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

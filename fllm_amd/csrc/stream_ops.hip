@@ -1,0 +1,132 @@
+// Small kernels on the residual stream and around the feed-forward that the dense decoder's own kernels do not
+// cover: two RMSNorms of one row in one pass (blocks whose branches read the same stream), a gated activation with
+// clamped operands, a vector and the embedding added to the stream between passes of looped layers, and logits times
+// a constant.  All arithmetic is float32; the element type only says how operands are stored.
+#include "api.h"
+#include "common.h"
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kWaves = kBlock / kWave;
+
+// One workgroup a row.  The sum of squares is added in a fixed order (thread t its columns t, t + 256, ..., then
+// lanes, then waves): a row gives the same bits whatever else is in the batch.  Both norms share the sum.
+template <typename T>
+__global__ void __launch_bounds__(kBlock)
+rmsnorm_pair_kernel(const float *__restrict__ x, const float *__restrict__ w1, const float *__restrict__ w2,
+                    T *__restrict__ out1, T *__restrict__ out2, int width, float eps1, float eps2) {
+    __shared__ float scratch[kWaves];
+    const size_t r = blockIdx.x;
+    const float *src = x + r * width;
+    float ss = 0.f;
+    for (int c = threadIdx.x; c < width; c += kBlock) ss += src[c] * src[c];
+    ss = block_sum<kWaves>(ss, scratch);
+    const float mean = ss / (float)width;
+    const float inv1 = 1.0f / sqrtf(mean + eps1), inv2 = 1.0f / sqrtf(mean + eps2);
+    for (int c = threadIdx.x; c < width; c += kBlock) {
+        const float v = src[c];
+        out1[r * width + c] = from_f32<T>(v * inv1 * w1[c]);
+        if (out2 != nullptr) out2[r * width + c] = from_f32<T>(v * inv2 * w2[c]);
+    }
+}
+
+// out = a(g) * (u + up_offset) with g = min(gate, limit), u = clamp(up, -limit, limit) (limit <= 0: neither is
+// clamped) and a(g) = g * sigmoid(alpha * g)
+template <typename T>
+__global__ void __launch_bounds__(kBlock)
+glu_clamped_kernel(const T *__restrict__ gu, T *__restrict__ out, int inter, float limit, float alpha, float up_offset) {
+    const size_t r = blockIdx.y;
+    const T *g = gu + r * 2 * inter, *u = g + inter;
+    T *o = out + r * inter;
+    const int c = blockIdx.x * kBlock + threadIdx.x;
+    if (c >= inter) return;
+    float gf = to_f32<T>(g[c]), uf = to_f32<T>(u[c]);
+    if (limit > 0.f) {
+        gf = fminf(gf, limit);
+        uf = fminf(fmaxf(uf, -limit), limit);
+    }
+    o[c] = from_f32<T>(gf / (1.0f + expf(-alpha * gf)) * (uf + up_offset));
+}
+
+__global__ void __launch_bounds__(kBlock) scale_kernel(float *__restrict__ x, size_t total, float scale) {
+    for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += (size_t)gridDim.x * kBlock) x[i] *= scale;
+}
+
+// x[r, :] = (x[r, :] + scale * table[ids[r], :]) + vec[:]; either addend may be absent
+template <typename T>
+__global__ void __launch_bounds__(kBlock)
+stream_add_kernel(float *__restrict__ x, const int32_t *__restrict__ ids, const T *__restrict__ table, int vocab, float scale,
+                  const float *__restrict__ vec, int width) {
+    const size_t r = blockIdx.x;
+    const T *src = nullptr;
+    if (table != nullptr) {
+        int id = ids[r];
+        id = id < 0 ? 0 : (id >= vocab ? vocab - 1 : id);   // ids are validated on the host; never read outside the table
+        src = table + (size_t)id * width;
+    }
+    float *dst = x + r * width;
+    for (int c = threadIdx.x; c < width; c += kBlock) {
+        float v = dst[c];
+        if (src != nullptr) v += to_f32<T>(src[c]) * scale;
+        if (vec != nullptr) v += vec[c];
+        dst[c] = v;
+    }
+}
+
+}  // namespace
+
+extern "C" int fllm_rmsnorm_pair(const float *x, const float *w1, const float *w2, void *out1, void *out2, int rows, int width,
+                                 float eps1, float eps2, int out_dtype, hipStream_t stream) {
+    FLLM_REQUIRE(rows >= 0 && width > 0, "rmsnorm_pair: bad sizes");
+    FLLM_REQUIRE(x && w1 && out1 && ((w2 == nullptr) == (out2 == nullptr)), "rmsnorm_pair: operands missing");
+    if (rows == 0) return 0;
+    if (out_dtype == FLLM_F32)
+        hipLaunchKernelGGL(rmsnorm_pair_kernel<float>, dim3(rows), dim3(kBlock), 0, stream, x, w1, w2, (float *)out1, (float *)out2,
+                           width, eps1, eps2);
+    else if (out_dtype == FLLM_BF16)
+        hipLaunchKernelGGL(rmsnorm_pair_kernel<bf16_t>, dim3(rows), dim3(kBlock), 0, stream, x, w1, w2, (bf16_t *)out1,
+                           (bf16_t *)out2, width, eps1, eps2);
+    else
+        FLLM_REQUIRE(false, "rmsnorm_pair: unknown dtype %d", out_dtype);
+    return fllm_check_launch("rmsnorm_pair");
+}
+
+extern "C" int fllm_glu_clamped(const void *gate_up, void *out, int rows, int inter, float limit, float alpha, float up_offset,
+                                int dtype, hipStream_t stream) {
+    FLLM_REQUIRE(rows >= 0 && inter > 0 && rows <= 65535, "glu_clamped: bad sizes");
+    if (rows == 0) return 0;
+    const dim3 grid((inter + kBlock - 1) / kBlock, rows);
+    if (dtype == FLLM_F32)
+        hipLaunchKernelGGL(glu_clamped_kernel<float>, grid, dim3(kBlock), 0, stream, (const float *)gate_up, (float *)out, inter,
+                           limit, alpha, up_offset);
+    else if (dtype == FLLM_BF16)
+        hipLaunchKernelGGL(glu_clamped_kernel<bf16_t>, grid, dim3(kBlock), 0, stream, (const bf16_t *)gate_up, (bf16_t *)out, inter,
+                           limit, alpha, up_offset);
+    else
+        FLLM_REQUIRE(false, "glu_clamped: unknown dtype %d", dtype);
+    return fllm_check_launch("glu_clamped");
+}
+
+extern "C" int fllm_scale_f32(float *x, size_t total, float scale, hipStream_t stream) {
+    if (total == 0) return 0;
+    const size_t blocks = (total + kBlock - 1) / kBlock;
+    hipLaunchKernelGGL(scale_kernel, dim3((unsigned)(blocks < 4096 ? blocks : 4096)), dim3(kBlock), 0, stream, x, total, scale);
+    return fllm_check_launch("scale_f32");
+}
+
+extern "C" int fllm_stream_add(float *x, const int32_t *ids, const void *table, int table_dtype, int vocab, float scale,
+                               const float *vec, int rows, int width, hipStream_t stream) {
+    FLLM_REQUIRE(rows >= 0 && width > 0, "stream_add: bad sizes");
+    FLLM_REQUIRE(table == nullptr || (ids != nullptr && vocab > 0), "stream_add: a table needs ids");
+    if (rows == 0 || (table == nullptr && vec == nullptr)) return 0;
+    if (table_dtype == FLLM_F32)
+        hipLaunchKernelGGL(stream_add_kernel<float>, dim3(rows), dim3(kBlock), 0, stream, x, ids, (const float *)table, vocab, scale,
+                           vec, width);
+    else if (table_dtype == FLLM_BF16)
+        hipLaunchKernelGGL(stream_add_kernel<bf16_t>, dim3(rows), dim3(kBlock), 0, stream, x, ids, (const bf16_t *)table, vocab,
+                           scale, vec, width);
+    else
+        FLLM_REQUIRE(false, "stream_add: unknown dtype %d", table_dtype);
+    return fllm_check_launch("stream_add");
+}

@@ -44,6 +44,8 @@ class Model:
             if layer.extras:            # only an arrangement that names further parts is handed them
                 placed["extras"] = {name: make(role, part) for name, (role, part) in layer.extras.items()}
             self.blocks.append(make("block", layer.block, **placed))
+        # what a run entry does to the stream before its layer (the input of a pass of looped layers)
+        self.before = [make("stream", entry.before) if entry.before is not None else None for entry in spec.run_order]
         self.final_norm = make("norm", spec.final_norm)
         self.head = make("head", spec.head)
         if consume_tensors:
@@ -180,12 +182,19 @@ class Model:
         order = self.spec.run_order
         for index, (entry, binding) in enumerate(zip(order, self.bindings)):
             block = self.blocks[entry.layer]
+            if self.before[index] is not None:
+                if pending is not None:
+                    self.rt.ops.add_residual(x, pending)
+                    pending = None
+                ctx.prepared = None              # the stream changes: whatever the block before prepared is void
+                self.before[index].forward(ctx, x, self.embedding)
             if check is not None:
                 check.run_block(self, block, ctx, x, binding, index, entry.layer)
                 continue
             # the norm that reads the residual stream after this block: the first one of the block that runs next,
             # where that block says which it is (a block may let its last sum prepare it)
-            ctx.next_norm = self.blocks[order[index + 1].layer].first_norm() if index + 1 < len(order) else None
+            ctx.next_norm = (self.blocks[order[index + 1].layer].first_norm()
+                             if index + 1 < len(order) and self.before[index + 1] is None else None)
             if getattr(block, "takes_pending", False):
                 pending = block.forward(ctx, x, binding, pending)
             else:

@@ -115,7 +115,8 @@ class ModelRunner:
         parts_ok = all(getattr(b.mixer, "graph_safe", False)
                        and (b.feed_forward is None or getattr(b.feed_forward, "graph_safe", False))
                        and all(getattr(p, "graph_safe", False) for p in getattr(b, "extras", {}).values())
-                       for b in self.model.blocks)
+                       for b in self.model.blocks) and all(p is None or getattr(p, "graph_safe", False)
+                                                            for p in self.model.before)
         self.use_graphs = bool(use_graphs) and self.device.type == "cuda" and parts_ok
         self._graphs: Dict[tuple, "_DecodeGraph"] = {}
         self._graph_pool = None

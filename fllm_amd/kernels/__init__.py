@@ -49,7 +49,7 @@ assert SAMPLE_ROW_BYTES == 32
 _lib = None
 
 
-ABI_VERSION = 11
+ABI_VERSION = 12
 
 
 def load_library(build_if_missing: bool = True):
@@ -106,6 +106,16 @@ def load_library(build_if_missing: bool = True):
         "fllm_adjust_logits": [c_void, c_int, c_int, c_void, c_void, c_void, c_void],
         "fllm_logprobs": [c_void, c_int, c_int, c_void, c_int, c_void, c_int, c_void, c_void, c_void],
         "fllm_logprobs_processed": [c_void, c_int, c_int, c_void, c_int, c_void, c_void, c_int, c_void, c_void, c_void],
+        "fllm_rmsnorm_pair": [c_void, c_void, c_void, c_void, c_void, c_int, c_int, c_float, c_float, c_int, c_void],
+        "fllm_glu_clamped": [c_void, c_void, c_int, c_int, c_float, c_float, c_float, c_int, c_void],
+        "fllm_scale_f32": [c_void, c_size, c_float, c_void],
+        "fllm_stream_add": [c_void, c_void, c_void, c_int, c_int, c_float, c_void, c_int, c_int, c_void],
+        "fllm_qk_norm_rope_store": [c_void, c_int, c_void, c_void, c_float, c_void, c_void, c_void, c_void, c_int, c_void, c_void,
+                                    c_int, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int,
+                                    c_void],
+        "fllm_talking_attention": [c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_void,
+                                   c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int,
+                                   c_void],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)
@@ -659,6 +669,127 @@ class Ops:
             _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(tables), tables.shape[1], _ptr(row_pos), _ptr(row_seg),
             _ptr(seg_start), seg_start.numel() - 1, _ptr(out), rows, heads, kv_heads, head_dim, page_size, num_pages, float(scale),
             int(window) if window else 0, _DTYPE_CODE[q.dtype], int(max_context), int(single_from), ws_ptr, ws_bytes,
+            self._stream()))
+        return out
+
+    # ---- parts of other layer designs ----------------------------------------------------------------------
+    def rmsnorm_pair(self, x: torch.Tensor, w1: torch.Tensor, eps1: float, out1: torch.Tensor,
+                     w2: Optional[torch.Tensor] = None, eps2: Optional[float] = None, out2: Optional[torch.Tensor] = None):
+        """Two RMSNorms of the same float32 rows in one pass over them (w2 and out2 None: one)."""
+        rows, width = x.shape
+        _dense(x, "x", torch.float32)
+        _dense(w1, "w1", torch.float32, (width,))
+        _dense(out1, "out1", None, (rows, width))
+        _need(out1.dtype in _DTYPE_CODE, f"out dtype {out1.dtype} unsupported")
+        _need((w2 is None) == (out2 is None), "the second norm needs a weight and an output")
+        if w2 is not None:
+            _dense(w2, "w2", torch.float32, (width,))
+            _dense(out2, "out2", out1.dtype, (rows, width))
+        self._check(self.lib.fllm_rmsnorm_pair(_ptr(x), _ptr(w1), _ptr(w2), _ptr(out1), _ptr(out2), rows, width, float(eps1),
+                                               float(eps1 if eps2 is None else eps2), _DTYPE_CODE[out1.dtype], self._stream()))
+        return out1, out2
+
+    def glu_clamped(self, gate_up: torch.Tensor, out: torch.Tensor, limit: float, alpha: float, up_offset: float) -> torch.Tensor:
+        """out = g * sigmoid(alpha * g) * (u + up_offset), g = min(gate, limit), u = clamp(up, -limit, limit) (limit <= 0:
+        nothing is clamped); gate_up = [gate | up] side by side in every row."""
+        rows, two_i = gate_up.shape
+        _need(two_i % 2 == 0, "gate_up needs an even width")
+        _dense(gate_up, "gate_up")
+        _need(gate_up.dtype in _DTYPE_CODE, f"dtype {gate_up.dtype} unsupported")
+        _dense(out, "out", gate_up.dtype, (rows, two_i // 2))
+        self._check(self.lib.fllm_glu_clamped(_ptr(gate_up), _ptr(out), rows, two_i // 2, float(limit), float(alpha),
+                                              float(up_offset), _DTYPE_CODE[gate_up.dtype], self._stream()))
+        return out
+
+    def scale_(self, x: torch.Tensor, scale: float) -> torch.Tensor:
+        """x *= scale, float32, in place."""
+        _dense(x, "x", torch.float32)
+        self._check(self.lib.fllm_scale_f32(_ptr(x), x.numel(), float(scale), self._stream()))
+        return x
+
+    def stream_add(self, x: torch.Tensor, ids: Optional[torch.Tensor] = None, table: Optional[torch.Tensor] = None,
+                   scale: float = 1.0, vec: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """x[r] = (x[r] + scale * table[ids[r]]) + vec: the embedding of the rows' tokens and / or one vector added to the
+        float32 residual stream."""
+        rows, width = x.shape
+        _dense(x, "x", torch.float32)
+        vocab, code = 0, F32
+        if table is not None:
+            _need(ids is not None, "a table needs ids")
+            _dense(ids, "ids", torch.int32, (rows,))
+            _dense(table, "table")
+            _need(table.dtype in _DTYPE_CODE and table.dim() == 2 and table.shape[1] == width, f"table must be [vocab, {width}]")
+            vocab, code = table.shape[0], _DTYPE_CODE[table.dtype]
+        if vec is not None:
+            _dense(vec, "vec", torch.float32, (width,))
+        self._check(self.lib.fllm_stream_add(_ptr(x), _ptr(ids) if table is not None else None, _ptr(table), code, vocab,
+                                             float(scale), _ptr(vec), rows, width, self._stream()))
+        return x
+
+    def _talking_pages(self, k_pages, v_pages, dtype, kv_heads, k_dim, v_dim, page_size, key_chunk):
+        _need(key_chunk > 0 and k_dim % key_chunk == 0, f"keys of {k_dim} values cannot lie in chunks of {key_chunk}")
+        num_pages = k_pages.shape[0]
+        _dense(k_pages, "k_pages", dtype, (num_pages, kv_heads, k_dim // key_chunk, page_size, key_chunk))
+        _dense(v_pages, "v_pages", dtype, (num_pages, kv_heads, v_dim, page_size))
+
+    def qk_norm_rope_store(self, qkv: torch.Tensor, q_weight: torch.Tensor, k_weight: torch.Tensor, eps: float, q_out: torch.Tensor,
+                           row_pos: torch.Tensor, row_seg: torch.Tensor, tables: torch.Tensor, cos: torch.Tensor, sin: torch.Tensor,
+                           k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor], heads: int, kv_heads: int, k_dim: int,
+                           v_dim: int, rope_dims: int, page_size: int, key_chunk: int) -> torch.Tensor:
+        """Rows of a joint product [q | k | v | ...]: RMSNorm over the whole query projection and over the whole key
+        projection, rotary on the first `rope_dims` lanes of every head (lane i with lane i + rope_dims / 2), queries to
+        `q_out`, keys and values into the pages (None: nothing is stored)."""
+        rows = qkv.shape[0]
+        _need(qkv.is_cuda and qkv.dim() == 2 and qkv.is_contiguous() and qkv.dtype in _DTYPE_CODE, "qkv must be dense rows on the GPU")
+        _need(qkv.shape[1] >= heads * k_dim + kv_heads * (k_dim + v_dim), "qkv rows are too short for q, k and v")
+        _dense(q_weight, "q_weight", torch.float32, (heads * k_dim,))
+        _dense(k_weight, "k_weight", torch.float32, (kv_heads * k_dim,))
+        _dense(q_out, "q_out", qkv.dtype, (rows, heads * k_dim))
+        _dense(row_pos, "row_pos", torch.int32, (rows,))
+        _dense(row_seg, "row_seg", torch.int32, (rows,))
+        _dense(tables, "tables", torch.int32)
+        _need(tables.dim() == 2, "tables must be [segments, pages]")
+        _dense(cos, "cos", torch.float32)
+        _dense(sin, "sin", torch.float32, tuple(cos.shape))
+        _need(cos.dim() == 2 and cos.shape[1] == rope_dims // 2, f"rotary tables must be [positions, {rope_dims // 2}]")
+        store = k_pages is not None
+        if store:
+            self._talking_pages(k_pages, v_pages, qkv.dtype, kv_heads, k_dim, v_dim, page_size, key_chunk)
+        self._check(self.lib.fllm_qk_norm_rope_store(
+            _ptr(qkv), qkv.shape[1], _ptr(q_weight), _ptr(k_weight), float(eps), _ptr(q_out), _ptr(row_pos), _ptr(row_seg),
+            _ptr(tables), tables.shape[1], _ptr(cos), _ptr(sin), cos.shape[0], _ptr(k_pages), _ptr(v_pages), rows, heads, kv_heads,
+            k_dim, v_dim, rope_dims, page_size, key_chunk, _DTYPE_CODE[qkv.dtype], 1 if store else 0, self._stream()))
+        return q_out
+
+    def talking_attention(self, q: torch.Tensor, gate: Optional[torch.Tensor], k_pages: torch.Tensor, v_pages: torch.Tensor,
+                          tables: torch.Tensor, row_pos: torch.Tensor, row_seg: torch.Tensor, seg_start: torch.Tensor,
+                          talk: torch.Tensor, temp: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int, k_dim: int,
+                          v_dim: int, page_size: int, scale: float, chunk: Optional[int], key_chunk: int, max_context: int) -> torch.Tensor:
+        """Attention whose scores are mixed across heads before the softmax (score[h] = sum_g talk[h, g] * q_g . k * scale *
+        temp[g]) over the keys of the row's own chunk of `chunk` positions up to the row (None: all keys up to the row);
+        head h's output times sigmoid(gate[row, h]) (`gate` may be a column slice of a wider matrix; None: no gate)."""
+        rows = q.shape[0]
+        _dense(q, "q", None, (rows, heads * k_dim))
+        _need(q.dtype in _DTYPE_CODE, f"dtype {q.dtype} unsupported")
+        gate_stride = 0
+        if gate is not None:
+            _need(gate.is_cuda and gate.dtype == q.dtype and tuple(gate.shape) == (rows, heads) and gate.stride(1) == 1,
+                  f"gate must be [rows, {heads}] of {q.dtype} with unit column stride")
+            gate_stride = gate.stride(0) if rows > 1 else heads
+        self._talking_pages(k_pages, v_pages, q.dtype, kv_heads, k_dim, v_dim, page_size, key_chunk)
+        _dense(tables, "tables", torch.int32)
+        _need(tables.dim() == 2, "tables must be [segments, pages]")
+        _dense(row_pos, "row_pos", torch.int32, (rows,))
+        _dense(row_seg, "row_seg", torch.int32, (rows,))
+        _dense(seg_start, "seg_start", torch.int32)
+        _need(seg_start.numel() >= 2 and tables.shape[0] >= seg_start.numel() - 1, "tables must have a row per segment")
+        _dense(talk, "talk", torch.float32, (heads, heads))
+        _dense(temp, "temp", torch.float32, (heads,))
+        _dense(out, "out", q.dtype, (rows, heads * v_dim))
+        self._check(self.lib.fllm_talking_attention(
+            _ptr(q), _ptr(gate), gate_stride, _ptr(k_pages), _ptr(v_pages), _ptr(tables), tables.shape[1], _ptr(row_pos),
+            _ptr(row_seg), _ptr(seg_start), seg_start.numel() - 1, _ptr(talk), _ptr(temp), _ptr(out), rows, heads, kv_heads, k_dim,
+            v_dim, page_size, float(scale), int(chunk) if chunk else 0, key_chunk, _DTYPE_CODE[q.dtype], int(max_context),
             self._stream()))
         return out
 

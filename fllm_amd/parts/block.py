@@ -1,5 +1,6 @@
 """Arrangement of parts in a layer.  `prenorm`: x += mixer(norm(x)); x += feed_forward(norm(x))
-(rust/engine/src/rust_decoder.rs:8764-8766, :9059-9088)."""
+(rust/engine/src/rust_decoder.rs:8764-8766, :9059-9088).  `parallel`: x += mixer(norm_a(x)) + feed_forward(norm_b(x)),
+both branches behind norms of their own of the same x."""
 from __future__ import annotations
 
 from ..registry import register_part
@@ -86,4 +87,36 @@ class PreNormBlock(Block):
         return None
 
 
+class ParallelBlock(Block):
+    """Both branches read the stream as the layer found it, each through its own norm; their outputs are added to it.
+    Where both norms are of the form x * rsqrt(mean x^2 + eps) * w they share one pass over the rows."""
+
+    def __init__(self, spec, weights, rt, mixer=None, feed_forward=None, norms=None):
+        super().__init__(spec, weights, rt)
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.mixer_norm = norms["mixer"]
+        self.feed_forward_norm = norms["feed_forward"] if feed_forward is not None else None
+
+    def forward(self, ctx, residual, binding):
+        rt, ops = self.rt, self.rt.ops
+        ctx.then_norm = ctx.prepared = None          # the sums of this block's parts are not read by a norm they know
+        first = getattr(self.mixer_norm, "fused_prologue", lambda: None)()
+        second = getattr(self.feed_forward_norm, "fused_prologue", lambda: None)() if self.feed_forward is not None else None
+        pair = getattr(ops, "rmsnorm_pair", None)
+        if self.feed_forward is None:
+            self.mixer.forward(ctx, self.mixer_norm.forward(ctx, residual), residual, binding)
+            return
+        if pair is not None and first is not None and second is not None:
+            h_mixer, h_ff = rt.empty(tuple(residual.shape)), rt.empty(tuple(residual.shape))
+            pair(residual, first[0], first[1], h_mixer, second[0], second[1], h_ff)
+        else:
+            h_mixer = self.mixer_norm.forward(ctx, residual)
+            h_ff = self.feed_forward_norm.forward(ctx, residual)
+        # both inputs exist before either branch adds to the stream
+        self.mixer.forward(ctx, h_mixer, residual, binding)
+        self.feed_forward.forward(ctx, h_ff, residual)
+
+
 register_part("block", "prenorm", PreNormBlock)
+register_part("block", "parallel", ParallelBlock)

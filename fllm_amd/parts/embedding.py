@@ -1,5 +1,5 @@
 """Token embedding (x[r] = scale * E[ids[r]], rust/engine/src/rust_decoder.rs:8605-8616) and
-the output head (logits = W h, float32; :8685)."""
+the output head (logits = W h, float32; :8685; times a constant where the model has one)."""
 from __future__ import annotations
 
 import torch
@@ -37,11 +37,15 @@ class LinearHead(Part):
         super().__init__(spec, weights, rt)
         self.weight = rt.matrix(weights["weight"])
         self.vocab = int(spec["vocab_size"])
+        self.scale = float(spec.get("scale", 1.0))       # logits = (W h) * scale, the product in float32
         rt.tile_for_decode(self.weight, priority=2)      # read once a step of up to 16 rows: after the layers' copies
 
     def forward(self, ctx, h):
         logits = self.rt.empty((h.shape[0], self.vocab), torch.float32)
-        return self.rt.ops.linear(h, self.weight, logits)
+        self.rt.ops.linear(h, self.weight, logits)
+        if self.scale != 1.0:
+            self.rt.ops.scale_(logits, self.scale)
+        return logits
 
 
 register_part("embedding", "table", TokenEmbedding)

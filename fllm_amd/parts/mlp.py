@@ -103,4 +103,36 @@ class GatedMLP(FeedForward):
         ops.linear(act, self.w_down, residual, bias=self.b_down, accumulate=True)
 
 
+class ClampedGLU(FeedForward):
+    """x += W_down (a(g) * (u + up_offset)) with g = min(W_gate n, limit), u = clamp(W_up n, -limit, limit) and
+    a(g) = g * sigmoid(alpha * g).  Gate and up are one product with the concatenated matrix."""
+    graph_safe = True
+
+    @classmethod
+    def tensor_shapes(cls, spec):
+        h, i = spec["hidden_size"], spec["intermediate_size"]
+        return {"gate": ((i, h), INIT_MATRIX), "up": ((i, h), INIT_MATRIX), "down": ((h, i), INIT_MATRIX)}
+
+    def __init__(self, spec, weights, rt):
+        super().__init__(spec, weights, rt)
+        self.hidden = int(spec["hidden_size"])
+        self.inter = int(spec["intermediate_size"])
+        self.limit = float(spec.get("limit") or 0.0)          # 0: nothing is clamped
+        self.alpha = float(spec.get("alpha", 1.0))
+        self.up_offset = float(spec.get("up_offset", 0.0))
+        self.w_gate_up = torch.cat([rt.matrix(weights["gate"]), rt.matrix(weights["up"])], dim=0).contiguous()
+        self.w_down = rt.matrix(weights["down"])
+        rt.tile_for_decode(self.w_down)
+
+    def forward(self, ctx, h, residual):
+        rt, ops = self.rt, self.rt.ops
+        rows = h.shape[0]
+        gate_up = rt.empty((rows, 2 * self.inter))
+        ops.linear(h, self.w_gate_up, gate_up)
+        act = rt.empty((rows, self.inter))
+        ops.glu_clamped(gate_up, act, self.limit, self.alpha, self.up_offset)
+        ops.linear(act, self.w_down, residual, accumulate=True)
+
+
 register_part("feed_forward", "gated_mlp", GatedMLP)
+register_part("feed_forward", "clamped_glu", ClampedGLU)

@@ -21,7 +21,7 @@ class Architecture:
 
 _ARCHITECTURES: Dict[str, Architecture] = {}
 _PARTS: Dict[str, Dict[str, type]] = {"mixer": {}, "feed_forward": {}, "norm": {}, "position": {}, "block": {},
-                                      "embedding": {}, "head": {}}
+                                      "embedding": {}, "head": {}, "stream": {}}
 
 
 def register_architecture(arch: Architecture) -> None:
@@ -36,6 +36,8 @@ def resolve_architecture(config: Dict[str, Any]) -> Architecture:
     """Dispatch on `model_type` (lower-cased), as the reference's decoders do
     (rust/checkpoint/src/plan.rs:880-884, :972-974); `architectures`, when present, must agree."""
     raw = config.get("model_type")
+    if raw is None and isinstance(config.get("architecture"), str):
+        raw = config["architecture"]          # files that name their design under `architecture` alone
     if not isinstance(raw, str) or not raw:
         raise ConfigError("config.json requires model_type")
     arch = _ARCHITECTURES.get(raw.lower())

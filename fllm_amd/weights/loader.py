@@ -40,6 +40,9 @@ def iter_parts(spec: ModelSpec):
         yield "block", layer.block
         for _, role, part in layer.parts():
             yield role, part
+    for entry in spec.run_order:
+        if entry.before is not None:
+            yield "stream", entry.before
     yield "norm", spec.final_norm
     yield "head", spec.head
 

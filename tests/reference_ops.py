@@ -153,6 +153,86 @@ class ReferenceOps:
                 out[r, h * head_dim:(h + 1) * head_dim] = (p @ v[:, h // group, :]).to(out.dtype)
         return out
 
+    # ---- parts of other layer designs: two norms of one row, clamped gated activation, what a pass of looped layers
+    # adds to the stream, logits times a constant, attention whose heads' scores are mixed before the softmax ----
+    def rmsnorm_pair(self, x, w1, eps1, out1, w2=None, eps2=None, out2=None):
+        self.rmsnorm(x, w1, eps1, out1)
+        if w2 is not None:
+            self.rmsnorm(x, w2, eps1 if eps2 is None else eps2, out2)
+        return out1, out2
+
+    def glu_clamped(self, gate_up, out, limit, alpha, up_offset):
+        inter = gate_up.shape[1] // 2
+        g, u = gate_up[:, :inter].double(), gate_up[:, inter:].double()
+        if limit > 0:
+            g, u = torch.clamp(g, max=limit), torch.clamp(u, -limit, limit)
+        out.copy_((g / (1.0 + torch.exp(-alpha * g)) * (u + up_offset)).to(out.dtype))
+        return out
+
+    def scale_(self, x, scale):
+        x.mul_(scale)
+        return x
+
+    def stream_add(self, x, ids=None, table=None, scale=1.0, vec=None):
+        y = x.double()
+        if table is not None:
+            y = y + table[ids.long()].double() * scale
+        if vec is not None:
+            y = y + vec.double()
+        x.copy_(y.to(x.dtype))
+        return x
+
+    def qk_norm_rope_store(self, qkv, q_weight, k_weight, eps, q_out, row_pos, row_seg, tables, cos, sin, k_pages, v_pages,
+                           heads, kv_heads, k_dim, v_dim, rope_dims, page_size, key_chunk):
+        nq, nk, nv = heads * k_dim, kv_heads * k_dim, kv_heads * v_dim
+        half = rope_dims // 2
+        for r in range(qkv.shape[0]):
+            seg = int(row_seg[r])
+            if seg < 0:
+                continue
+            pos = int(row_pos[r])
+            q, k = qkv[r, :nq].double(), qkv[r, nq:nq + nk].double()
+            q = (q / torch.sqrt((q * q).mean() + eps) * q_weight.double()).view(heads, k_dim).clone()
+            k = (k / torch.sqrt((k * k).mean() + eps) * k_weight.double()).view(kv_heads, k_dim).clone()
+            if half:
+                c, s = cos[pos].double(), sin[pos].double()
+                for t in (q, k):
+                    a, b = t[:, :half].clone(), t[:, half:rope_dims].clone()
+                    t[:, :half] = a * c - b * s
+                    t[:, half:rope_dims] = b * c + a * s
+            q_out[r] = q.reshape(-1).to(q_out.dtype)
+            if k_pages is None:
+                continue
+            page, off = int(tables[seg, pos // page_size]), pos % page_size
+            k_pages[page, :, :, off, :] = k.view(kv_heads, k_dim // key_chunk, key_chunk).to(k_pages.dtype)
+            v_pages[page, :, :, off] = qkv[r, nq + nk:nq + nk + nv].view(kv_heads, v_dim)
+        return q_out
+
+    def talking_attention(self, q, gate, k_pages, v_pages, tables, row_pos, row_seg, seg_start, talk, temp, out, heads, kv_heads,
+                          k_dim, v_dim, page_size, scale, chunk, key_chunk, max_context):
+        group = heads // kv_heads
+        for r in range(q.shape[0]):
+            seg = int(row_seg[r])
+            if seg < 0:
+                out[r] = 0
+                continue
+            pos = int(row_pos[r])
+            lo = pos - pos % chunk if chunk else 0
+            keys = torch.arange(lo, pos + 1, device=q.device)
+            pages = tables[seg, (keys // page_size).long()].long()
+            offs = (keys % page_size).long()
+            k = k_pages[pages, :, :, offs, :].double().reshape(len(keys), kv_heads, k_dim)
+            v = v_pages[pages, :, :, offs].double()                                    # [n, kv_heads, v_dim]
+            qr = q[r].double().view(heads, k_dim)
+            raw = torch.stack([(k[:, h // group, :] @ qr[h]) * scale * float(temp[h]) for h in range(heads)])    # [heads, n]
+            p = torch.softmax(talk.double() @ raw, dim=1)
+            for h in range(heads):
+                o = p[h] @ v[:, h // group, :]
+                if gate is not None:
+                    o = o / (1.0 + torch.exp(-gate[r, h].double()))
+                out[r, h * v_dim:(h + 1) * v_dim] = o.to(out.dtype)
+        return out
+
     def carry_ids(self, ids, source, previous):
         for r in range(ids.numel()):
             if int(source[r]) >= 0:

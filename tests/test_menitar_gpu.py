@@ -1,0 +1,436 @@
+"""Menitar on the MI355X: each of its kernels alone against tests/reference_ops.py (float64), then the engine's steps
+however a request is cut and batched, captured decode steps and greedy generation against tests/plain_menitar.py."""
+
+import numpy as np
+import pytest
+import torch
+
+import menitar_configs as mc
+import plain_menitar
+import trace_tools as tt
+from reference_ops import ReferenceOps
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+BF16_EPS = 2.0 ** -8
+
+
+@pytest.fixture(scope="module")
+def ops():
+    from fllm_amd.kernels import Ops
+    return Ops()
+
+
+@pytest.fixture(scope="module")
+def ref():
+    return ReferenceOps()
+
+
+def gen(seed):
+    g = torch.Generator()
+    g.manual_seed(seed)
+    return g
+
+
+def close(got, want, rtol, atol, what=""):
+    got, want = got.detach().double().cpu(), want.detach().double().cpu()
+    err = (got - want).abs()
+    worst = (err - (atol + rtol * want.abs())).max().item()
+    assert worst <= 0, f"{what}: max err {err.max().item():.3e} (|want| max {want.abs().max().item():.3e}), over by {worst:.3e}"
+
+
+# ---------------------------------------------------------------------------------------------
+# the small kernels
+# ---------------------------------------------------------------------------------------------
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("rows,width", [(1, 64), (7, 200), (33, 1000), (130, 4096)])
+def test_two_norms_of_one_row(ops, ref, rows, width, out_dtype):
+    x = torch.randn(rows, width, generator=gen(1)) * 3
+    w1, w2 = 1 + 0.3 * torch.randn(width, generator=gen(2)), 1 + 0.3 * torch.randn(width, generator=gen(3))
+    want1, want2 = torch.empty(rows, width, dtype=torch.float64), torch.empty(rows, width, dtype=torch.float64)
+    ref.rmsnorm_pair(x.double(), w1, 1e-5, want1, w2, 1e-3, want2)
+    got1, got2 = (torch.empty(rows, width, dtype=out_dtype, device=DEV) for _ in range(2))
+    ops.rmsnorm_pair(x.to(DEV), w1.to(DEV), 1e-5, got1, w2.to(DEV), 1e-3, got2)
+    tol = 2e-6 if out_dtype == torch.float32 else BF16_EPS
+    close(got1, want1, tol, 1e-6, "first norm")
+    close(got2, want2, tol, 1e-6, "second norm")
+    only = torch.empty(rows, width, dtype=out_dtype, device=DEV)
+    ops.rmsnorm_pair(x.to(DEV), w2.to(DEV), 1e-3, only)
+    assert torch.equal(only, got2)
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("limit,alpha,offset", [(1.5, 1.702, 1.0), (0.5, 1.0, 0.0), (0.0, 1.702, 1.0)])
+@pytest.mark.parametrize("rows,inter", [(1, 24), (9, 333), (70, 2048)])
+def test_clamped_gated_activation(ops, ref, rows, inter, limit, alpha, offset, dtype):
+    gate_up = (torch.randn(rows, 2 * inter, generator=gen(4)) * 2).to(dtype)      # many values beyond either limit
+    want = torch.empty(rows, inter, dtype=torch.float64)
+    ref.glu_clamped(gate_up.double(), want, limit, alpha, offset)
+    got = torch.empty(rows, inter, dtype=dtype, device=DEV)
+    ops.glu_clamped(gate_up.to(DEV), got, limit, alpha, offset)
+    close(got, want, 3e-6 if dtype == torch.float32 else BF16_EPS, 1e-6, "activation")
+
+
+@pytest.mark.parametrize("table_dtype", [torch.float32, torch.bfloat16])
+def test_what_a_pass_adds_to_the_stream(ops, ref, table_dtype):
+    rows, width, vocab = 37, 200, 90
+    x = torch.randn(rows, width, generator=gen(5))
+    table = torch.randn(vocab, width, generator=gen(6)).to(table_dtype)
+    vec = torch.randn(width, generator=gen(7))
+    ids = torch.randint(0, vocab, (rows,), generator=gen(8), dtype=torch.int32)
+    for use_table, use_vec in ((True, True), (True, False), (False, True)):
+        want = x.double().clone()
+        ref.stream_add(want, ids if use_table else None, table if use_table else None, 2.5, vec if use_vec else None)
+        got = x.to(DEV).clone()
+        ops.stream_add(got, ids.to(DEV) if use_table else None, table.to(DEV) if use_table else None, 2.5,
+                       vec.to(DEV) if use_vec else None)
+        close(got, want, 1e-6, 1e-6, f"stream_add table={use_table} vec={use_vec}")
+    y = x.to(DEV).clone()
+    ops.scale_(y, 0.37)
+    close(y, x.double() * 0.37, 1e-6, 0, "scale")
+
+
+# ---------------------------------------------------------------------------------------------
+# norm + rotary + store, and the attention, over scattered pages
+# ---------------------------------------------------------------------------------------------
+class Scene:
+    """Requests with `held` tokens in the cache and `new` rows in this step, pages dealt out in a shuffled order, caches
+    full of random numbers (so a key that must not be seen is loud, not zero)."""
+
+    def __init__(self, segs, H, G, d, dv, page, rope_dims, seed, dtype, loud=None):
+        g = gen(seed)
+        self.H, self.G, self.d, self.dv, self.page, self.rope_dims = H, G, d, dv, page, rope_dims
+        self.key_chunk = 8 if d % 8 == 0 else 1
+        longest = max(h + n for h, n in segs)
+        per_seg = -(-longest // page) + 1
+        num_pages = per_seg * len(segs) + 3
+        order = torch.randperm(num_pages, generator=g)[:per_seg * len(segs)].to(torch.int32)
+        self.tables = order.view(len(segs), per_seg).contiguous()
+        self.k_pages = torch.randn(num_pages, G, d // self.key_chunk, page, self.key_chunk, generator=g).to(dtype)
+        self.v_pages = torch.randn(num_pages, G, dv, page, generator=g).to(dtype)
+        pos, seg, start = [], [], [0]
+        for s, (held, new) in enumerate(segs):
+            pos += list(range(held, held + new))
+            seg += [s] * new
+            start.append(start[-1] + new)
+        self.row_pos = torch.tensor(pos, dtype=torch.int32)
+        self.row_seg = torch.tensor(seg, dtype=torch.int32)
+        self.seg_start = torch.tensor(start, dtype=torch.int32)
+        rows = len(pos)
+        width = H * d + G * (d + dv) + H
+        self.width = width + (-width) % 8
+        self.qkvg = torch.randn(rows, self.width, generator=g).to(dtype)
+        self.q_weight = 1 + 0.4 * torch.randn(H * d, generator=g)
+        self.k_weight = 1 + 0.4 * torch.randn(G * d, generator=g)
+        self.talk = torch.eye(H) + 0.4 * torch.randn(H, H, generator=g)
+        self.temp = 0.5 + 2 * torch.rand(H, generator=g)
+        half = rope_dims // 2
+        self.max_pos = longest + 1
+        freq = torch.tensor([500.0 ** (-2.0 * i / max(rope_dims, 1)) for i in range(half)], dtype=torch.float64)
+        angle = torch.arange(self.max_pos, dtype=torch.float64)[:, None] * freq[None, :]
+        self.cos, self.sin = torch.cos(angle).float(), torch.sin(angle).float()
+        if loud:            # (segment, position, factor): a cached key that would take all the weight of whoever sees it
+            for s, p, factor in loud:
+                self.k_pages[int(self.tables[s, p // page]), :, :, p % page, :] *= factor
+
+    def tensors(self, device, dtype=None):
+        names = ["tables", "k_pages", "v_pages", "row_pos", "row_seg", "seg_start", "qkvg", "q_weight", "k_weight", "talk",
+                 "temp", "cos", "sin"]
+        out = {n: getattr(self, n).clone().to(device) for n in names}
+        if dtype is not None:
+            for n in ("k_pages", "v_pages", "qkvg"):
+                out[n] = out[n].to(dtype)
+        return out
+
+
+def run_mixer_kernels(o, t, sc, chunk, scale, dtype):
+    rows = t["qkvg"].shape[0]
+    H, G, d, dv = sc.H, sc.G, sc.d, sc.dv
+    q = torch.empty(rows, H * d, dtype=dtype, device=t["qkvg"].device)
+    o.qk_norm_rope_store(t["qkvg"], t["q_weight"], t["k_weight"], 1e-5, q, t["row_pos"], t["row_seg"], t["tables"], t["cos"],
+                         t["sin"], t["k_pages"], t["v_pages"], H, G, d, dv, sc.rope_dims, sc.page, sc.key_chunk)
+    out = torch.empty(rows, H * dv, dtype=dtype, device=q.device)
+    gate_at = H * d + G * (d + dv)
+    o.talking_attention(q, t["qkvg"][:, gate_at:gate_at + H], t["k_pages"], t["v_pages"], t["tables"], t["row_pos"], t["row_seg"],
+                        t["seg_start"], t["talk"], t["temp"], out, H, G, d, dv, sc.page, scale, chunk, sc.key_chunk, sc.max_pos)
+    return q, out
+
+
+# heads, kv heads, key size, value size, chunk, page, rotated lanes
+SHAPES = [(4, 2, 32, 16, 24, 8, 16), (6, 3, 64, 64, 40, 16, 32), (12, 4, 32, 16, 16, 16, 32), (2, 1, 20, 12, None, 8, 0),
+          (8, 2, 64, 32, 80, 16, 32), (16, 16, 32, 32, 33, 32, 8), (3, 3, 32, 32, 40, 16, 32), (5, 1, 128, 128, 100, 64, 64),
+          (8, 8, 256, 64, None, 16, 64)]
+# (held, new) per request: prompts from the first token, portions that begin inside a chunk and cross its edge, single
+# rows right before, on and after an edge, two-token portions
+SEGMENTS = [(0, 50), (37, 1), (23, 30), (79, 2), (80, 1), (95, 18), (0, 1), (120, 1), (47, 1), (48, 1), (2, 2), (199, 1)]
+
+
+@pytest.mark.parametrize("fast", [True, False])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("shape", SHAPES)
+def test_mixed_head_attention_over_pages(ops, ref, shape, dtype, fast):
+    H, G, d, dv, chunk, page, rope_dims = shape
+    if dtype == torch.float32 and not fast:
+        pytest.skip("float32 has one kernel")
+    scale = d ** -0.5 * 1.3
+    # loud keys at the edges of what a row may see: the last position of the chunk before its own, and the position after
+    # itself (a stale key of a page that was used before)
+    loud = []
+    for s, (held, new) in enumerate(SEGMENTS):
+        last = held + new - 1
+        if chunk and last - last % chunk > 0 and held > 0:
+            loud.append((s, min(last - last % chunk, held) - 1, 8.0))
+        loud.append((s, last + 1, 8.0))
+    sc = Scene(SEGMENTS, H, G, d, dv, page, rope_dims, seed=H * 100 + d, dtype=dtype, loud=loud)
+    want_t = sc.tensors("cpu", torch.float64)
+    want_q, want = run_mixer_kernels(ref, want_t, sc, chunk, scale, torch.float64)
+    ops.set_fast_kernels(fast)
+    try:
+        got_t = sc.tensors(DEV)
+        got_q, got = run_mixer_kernels(ops, got_t, sc, chunk, scale, dtype)
+        torch.cuda.synchronize()
+    finally:
+        ops.set_fast_kernels(True)
+    if dtype == torch.float32:
+        close(got_q, want_q, 1e-5, 1e-5, "queries")
+        close(got_t["k_pages"], want_t["k_pages"], 1e-5, 1e-5, "stored keys")
+        assert torch.equal(got_t["v_pages"].cpu().double(), want_t["v_pages"])
+        close(got, want, 5e-4, 5e-4, "attention")
+    else:
+        close(got_q, want_q, BF16_EPS, 1e-3, "queries")
+        close(got_t["k_pages"], want_t["k_pages"], BF16_EPS, 1e-3, "stored keys")
+        assert torch.equal(got_t["v_pages"].cpu().double(), want_t["v_pages"])
+        # the reference continues from its own float64 queries and keys; sharp softmaxes amplify the rounding of the
+        # bfloat16 ones, so the kernel is held against the reference run on what the kernel itself stored
+        again = sc.tensors("cpu", torch.float64)
+        again["k_pages"], again["v_pages"] = got_t["k_pages"].cpu().double(), got_t["v_pages"].cpu().double()
+        want2 = torch.empty_like(want)
+        gate_at = H * d + G * (d + dv)
+        ref.talking_attention(got_q.cpu().double(), again["qkvg"][:, gate_at:gate_at + H], again["k_pages"], again["v_pages"],
+                              again["tables"], again["row_pos"], again["row_seg"], again["seg_start"], again["talk"].double(),
+                              again["temp"].double(), want2, H, G, d, dv, page, scale, chunk, sc.key_chunk, sc.max_pos)
+        close(got, want2, 3 * BF16_EPS, 3e-2, "attention")
+
+
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("where", ["first of the chunk", "just outside", "far back", "itself"])
+def test_one_key_that_stands_out(ops, ref, where, dtype):
+    """One key among hundreds takes nearly all the weight of one head: the output is that key's value when the row may see
+    it, and shows no trace of it when the key lies one position outside the row's chunk."""
+    H, G, d, dv, chunk, page = 4, 2, 64, 32, 100, 16
+    held = 100 * 3 + 40                                   # the row at position 340 sees 300 .. 340
+    lo = held - held % chunk
+    target = {"first of the chunk": lo, "just outside": lo - 1, "far back": 5, "itself": held}[where]
+    sc = Scene([(held, 1), (7, 3)], H, G, d, dv, page, 0, seed=9, dtype=dtype)
+    t = sc.tensors(DEV)
+    # identity mixing, unit temperatures: head h's score is q_h . k; make q of head 1 and key `target` (kv head 0) long
+    # and parallel
+    t["talk"] = torch.eye(H, device=DEV)
+    t["temp"] = torch.ones(H, device=DEV)
+    rows = t["qkvg"].shape[0]
+    q = (0.05 * torch.randn(rows, H * d, generator=gen(3))).to(dtype).to(DEV)
+    direction = torch.randn(d, generator=gen(4))
+    direction = (direction / direction.norm()).to(dtype)
+    q[0, d:2 * d] = (direction.float() * 8).to(dtype).to(DEV)
+    t["k_pages"].mul_(0.05)
+    gate = torch.full((rows, H), 20.0, dtype=dtype, device=DEV)          # sigmoid = 1
+    # (the row's own key is written by the store kernel in a model; here every key is placed by hand)
+    pg, off = int(sc.tables[0, target // page]), target % page
+    t["k_pages"][pg, 0, :, off, :] = (direction.float() * 8).view(d // 8, 8).to(dtype).to(DEV)
+    out = torch.empty(rows, H * dv, dtype=dtype, device=DEV)
+    ops.talking_attention(q, gate, t["k_pages"], t["v_pages"], t["tables"], t["row_pos"], t["row_seg"], t["seg_start"],
+                          t["talk"], t["temp"], out, H, G, d, dv, page, 1.0, chunk, sc.key_chunk, sc.max_pos)
+    head1 = out[0, dv:2 * dv].float().cpu()
+    value = t["v_pages"][pg, 0, :, off].float().cpu()
+    seen = lo <= target <= held
+    if seen:
+        close(head1, value, 2 * BF16_EPS, 2e-2, where)
+    else:
+        assert (head1 - value).abs().max() > 0.3, f"{where}: the key must not be seen"
+        quiet = t["k_pages"].clone()
+        quiet[pg, 0, :, off, :] = 0
+        out2 = torch.empty_like(out)
+        ops.talking_attention(q, gate, quiet, t["v_pages"], t["tables"], t["row_pos"], t["row_seg"], t["seg_start"],
+                              t["talk"], t["temp"], out2, H, G, d, dv, page, 1.0, chunk, sc.key_chunk, sc.max_pos)
+        assert torch.equal(out, out2), f"{where}: a key outside the chunk changed the output"
+
+
+def test_the_matrix_core_kernel_is_the_one_that_runs(ops):
+    """bfloat16 with heads of a multiple of 32 values runs the matrix-core kernel: the plain one, switched on instead, rounds
+    differently somewhere."""
+    H, G, d, dv, chunk, page = 6, 3, 64, 64, 40, 16
+    sc = Scene(SEGMENTS, H, G, d, dv, page, 32, seed=77, dtype=torch.bfloat16)
+    outs = []
+    for fast in (True, False):
+        ops.set_fast_kernels(fast)
+        try:
+            outs.append(run_mixer_kernels(ops, sc.tensors(DEV), sc, chunk, 0.2, torch.bfloat16)[1].float().cpu())
+        finally:
+            ops.set_fast_kernels(True)
+    assert not torch.equal(outs[0], outs[1])
+    close(outs[0], outs[1], 4 * BF16_EPS, 4e-2, "two kernels")
+
+
+# ---------------------------------------------------------------------------------------------
+# the engine
+# ---------------------------------------------------------------------------------------------
+LENGTHS = {"P": [5, 30, 61, 100, 49], "Q": [45, 83, 161, 2, 120], "R": [9, 50, 300, 130], "S": [100, 37, 250, 81, 160],
+           "T": [3, 17, 64, 33, 150]}
+# about three times the largest error any case here has shown on the MI355X (float32 8.4e-7, bfloat16 8.6e-3)
+TOL = {"float32": 3e-6, "bfloat16": 2.5e-2}
+
+
+@pytest.fixture(scope="module")
+def models(tmp_path_factory):
+    out = {}
+    for name, cfg in mc.CONFIGS.items():
+        tensors = mc.weights(cfg, 30 + ord(name))
+        folder = mc.write_model(str(tmp_path_factory.mktemp(f"menitar_{name}")), cfg, tensors)
+        requests = {f"r{i}": mc.random_ids(n, cfg["vocab"], 100 * ord(name) + i) for i, n in enumerate(LENGTHS[name])}
+        w64 = mc.to_float64(tensors)
+        plain = {rid: plain_menitar.forward(cfg, w64, toks) for rid, toks in requests.items()}
+        out[name] = (folder, cfg, requests, plain, w64)
+    return out
+
+
+def make_runner(folder, dtype, page_size, max_tokens, **kw):
+    from fllm_amd.engine import ModelRunner
+    return ModelRunner.from_folder(folder, dtype=dtype, page_size=page_size, max_tokens=max_tokens, max_requests=4, **kw)
+
+
+def check(got, plain, dtype, what):
+    for rid, want in plain.items():
+        assert rid in got and got[rid].shape == want.shape, f"{what}: request {rid}"
+        err = np.abs(got[rid].astype(np.float64) - want)
+        scale = np.abs(want).max()
+        tt.observe(f"menitar {what.split()[0]} {dtype}", err.max() / scale)
+        over = err.max(axis=1) > TOL[dtype] * scale
+        assert not over.any(), (f"{what}: request {rid}: max error {err.max():.3e} (limit {TOL[dtype] * scale:.3e}); first "
+                                f"position over the limit: {int(np.argmax(over))}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["P", "Q", "R", "S", "T"])
+@pytest.mark.parametrize("family", ["whole", "last40", "portions", "mixed"])
+def test_replay(models, tmp_path, name, dtype, family):
+    folder, cfg, requests, plain, _ = models[name]
+    refed = [rid for rid, toks in requests.items() if len(toks) >= 60][:1]
+    steps = {"whole": tt.whole, "last40": lambda r: tt.last_tokens_one_by_one(r, 40), "portions": tt.portions,
+             "mixed": lambda r: tt.mixed(r, seed=5, refeed=refed)}[family](requests)
+    steps = tt.number(steps)
+    runner = make_runner(folder, dtype, mc.PAGE_SIZES[name], tt.live_tokens_bound(steps))
+    handed_out = tt.record_allocations(runner.cache)
+    given_up = {}
+    got = tt.run_in_process(runner, steps, cfg["vocab"], str(tmp_path), given_up)
+    check(got, plain, dtype, f"{family} {name} {dtype}")
+    if family == "mixed" and dtype == "float32":
+        for rid, feedings in given_up.items():
+            for first in feedings:
+                assert np.array_equal(first, got[rid][:len(first)]), f"{rid}: fed again on other pages, other logits"
+    runner.cache.check_invariants()
+    assert all(pool.available == pool.num_pages for pool in runner.cache.pools), "pages were lost"
+    for pages in handed_out:
+        assert len(pages) > len(set(pages)), "the trace was meant to use pages again"
+
+
+@pytest.mark.parametrize("page_size", [4, 32, 64])
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_replay_at_other_page_sizes(models, tmp_path, page_size, dtype):
+    folder, cfg, requests, plain, _ = models["S"]
+    steps = tt.number(tt.mixed(requests, seed=8))
+    runner = make_runner(folder, dtype, page_size, tt.live_tokens_bound(steps, round_to=max(64, page_size)))
+    got = tt.run_in_process(runner, steps, cfg["vocab"], str(tmp_path))
+    check(got, plain, dtype, f"pages-of-{page_size} S {dtype}")
+
+
+def test_cuts_agree_bit_for_bit_in_float32(models, tmp_path):
+    folder, cfg, requests, plain, _ = models["P"]
+    results = []
+    for i, make in enumerate([tt.whole, tt.portions, lambda r: tt.mixed(r, seed=3)]):
+        steps = tt.number(make(requests))
+        runner = make_runner(folder, "float32", 8, tt.live_tokens_bound(steps))
+        results.append(tt.run_in_process(runner, steps, cfg["vocab"], str(tmp_path / str(i))))
+    for rid in requests:
+        assert np.array_equal(results[0][rid], results[1][rid]), f"whole vs portions differ for {rid}"
+        assert np.array_equal(results[0][rid], results[2][rid]), f"whole vs mixed differ for {rid}"
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["Q", "R"])
+def test_first_tokens_and_long_decoding(models, tmp_path, name, dtype):
+    """Token by token from the very first token, across several chunks of positions (Q) and with every key seen (R)."""
+    folder, cfg, requests, plain, _ = models[name]
+    rid = "r2"
+    one = {rid: requests[rid]}
+    steps = tt.number(tt.last_tokens_one_by_one(one, tail=len(requests[rid])))
+    runner = make_runner(folder, dtype, mc.PAGE_SIZES[name], 320)
+    got = tt.run_in_process(runner, steps, cfg["vocab"], str(tmp_path))
+    check(got, {rid: plain[rid]}, dtype, f"token-by-token {name} {dtype}")
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["P", "S"])
+def test_decode_graphs_and_eager_steps_agree(models, tmp_path, name, dtype):
+    folder, cfg, requests, plain, _ = models[name]
+    steps = tt.number(tt.last_tokens_one_by_one(requests) + tt.mixed(requests, seed=21, decode_tail=40))
+    results = []
+    for i, use_graphs in enumerate((True, False)):
+        runner = make_runner(folder, dtype, mc.PAGE_SIZES[name], tt.live_tokens_bound(steps), use_graphs=use_graphs)
+        results.append(tt.run_in_process(runner, steps, cfg["vocab"], str(tmp_path / str(i))))
+        assert (runner.graph_replays > 30) == use_graphs
+    for rid, want in plain.items():
+        a, b = results[0][rid].astype(np.float64), results[1][rid].astype(np.float64)
+        if dtype == "float32":
+            assert np.array_equal(a, b), f"{rid}: graph and eager steps differ in float32"
+        else:
+            assert np.abs(a - b).max() <= TOL[dtype] * np.abs(want).max()
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_trace_run_program(models, tmp_path, dtype):
+    folder, cfg, requests, plain, _ = models["S"]
+    steps = tt.number(tt.mixed(requests, seed=9))
+    got = tt.run_subprocess(folder, dtype, steps, cfg["vocab"], str(tmp_path), tt.live_tokens_bound(steps))
+    check(got, plain, dtype, f"trace_run S {dtype}")
+
+
+def test_the_residual_stream_after_every_layer_run(models):
+    folder, cfg, requests, plain, w64 = models["S"]
+    runner = make_runner(folder, "float32", 16, 320)
+    from fllm_amd.engine import StepEntry
+    seen = []
+    for block in runner.model.blocks:
+        def wrapped(ctx, x, binding, _inner=block.forward):
+            _inner(ctx, x, binding)
+            seen.append(x.clone().cpu().numpy())
+        block.forward = wrapped
+    toks = requests["r0"]
+    runner.step([StepEntry("a", toks, [])])
+    want = []
+    plain_menitar.forward(cfg, w64, toks, want)
+    assert len(seen) == len(want) == 5
+    for got, ref_x in zip(seen, want):
+        assert np.abs(got - ref_x).max() <= 1e-5 * np.abs(ref_x).max()
+
+
+@pytest.mark.parametrize("name", ["P", "S", "T"])
+def test_greedy_generation_through_the_scheduler(models, name):
+    from fllm_amd import Engine, SamplingParams
+    folder, cfg, _, _, w64 = models[name]
+    prompts = [mc.random_ids(n, cfg["vocab"], 20 + n) for n in (3, 26, 41, 90)]
+    want = [plain_menitar.greedy(cfg, w64, p, 12) for p in prompts]
+    for opts in (dict(num_blocks=64), dict(num_blocks=14, max_batched_tokens=16)):
+        engine = Engine(folder, dtype="float32", ctx=256, max_seqs=3, block_size=mc.PAGE_SIZES[name],
+                        **{"max_batched_tokens": 64, **opts})
+        assert engine.generate(prompts, SamplingParams(max_tokens=12)) == want
+        engine.runner.cache.check_invariants()
+    engine = Engine(folder, dtype="bfloat16", ctx=256, max_seqs=4, block_size=mc.PAGE_SIZES[name])
+    out = engine.generate(prompts, SamplingParams(max_tokens=12))
+    assert [len(o) for o in out] == [12] * 4
+    # bfloat16 picks the same token wherever the plain logits leave a clear margin: the first token of every prompt
+    for p, o in zip(prompts, out):
+        logits = plain_menitar.forward(cfg, w64, p)[-1]
+        top = np.sort(logits)[-2:]
+        if top[1] - top[0] > 0.1 * np.abs(logits).max():
+            assert o[0] == int(np.argmax(logits))

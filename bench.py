@@ -202,6 +202,115 @@ def kernel_breakdown(run_steps, steps, top=8):
     return out or None
 
 
+# ---- another design beside the closest existing one, at equal sizes (--design) ------------------------------------------
+# layer sizes that resemble published models of 12 and 16 query heads of 128 (1.5B and 3B parameter class) and a small one
+DESIGN_SIZES = {
+    "small": dict(width=1024, heads=8, kv_heads=2, dim=128, ff=4096, layers=12, vocab=32768),
+    "1.5b": dict(width=1536, heads=12, kv_heads=2, dim=128, ff=8960, layers=28, vocab=151936),
+    "3b": dict(width=2048, heads=16, kv_heads=2, dim=128, ff=11008, layers=36, vocab=151936),
+}
+DESIGN_CHUNK = 8192          # positions see their own chunk of this many: at the contexts measured here, every earlier key
+
+
+def menitar_config(size, layers):
+    """`layers` layers of which the middle half runs twice (3 layers: 4 layer runs)."""
+    mixer = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["dim"],
+             "scale": size["dim"] ** -0.5, "rot": {"dims": size["dim"] // 2, "base": 10000.0}, "mask": {"size": DESIGN_CHUNK}}
+    layer = {"type": "attention", "mixer": mixer, "mlp": {"kind": "dense", "ff": size["ff"], "limit": 7.0}}
+    cfg = {"architecture": "Menitar", "width": size["width"], "vocab": size["vocab"], "embedding": {"scale": 1.0},
+           "logit_scale": 1.0, "norm": {"eps": 1e-5}, "layers": [layer] * layers, "max_position": 32768}
+    start, stop = layers // 4, layers // 4 + max(1, layers // 2)
+    if stop <= layers and layers >= 3:
+        cfg["loop"] = {"start": start, "stop": stop, "times": 2}
+        return cfg, layers + (stop - start)
+    return cfg, layers
+
+
+def llama_config_of(size, layer_runs):
+    return {"model_type": "llama", "architectures": ["LlamaForCausalLM"], "num_hidden_layers": layer_runs,
+            "hidden_size": size["width"], "num_attention_heads": size["heads"], "num_key_value_heads": size["kv_heads"],
+            "head_dim": size["dim"], "intermediate_size": size["ff"], "vocab_size": size["vocab"], "rope_theta": 10000.0,
+            "rms_norm_eps": 1e-5, "tie_word_embeddings": True, "max_position_embeddings": 32768, "hidden_act": "silu"}
+
+
+def design_run(args):
+    """Prefill and decode throughput of the Menitar design beside Llama at equal sizes (width, heads, head size,
+    feed-forward, vocabulary, as many layers as the other has layer runs), random bfloat16 weights, with the device time
+    of the kernels of a decode step and of a prefill step of each.  Prints one JSON line of its own."""
+    import gc
+    import numpy as np
+    import torch
+    from fllm_amd import Engine, SamplingParams
+    size = DESIGN_SIZES[args.design_size]
+    layers = args.layers or size["layers"]
+    menitar, layer_runs = menitar_config(size, layers)
+    models = {"menitar": (menitar, size["vocab"]), "llama": (llama_config_of(size, layer_runs), size["vocab"])}
+    batches = sorted({1, args.batch, 64})
+    steps, warmup = min(args.steps, 96), args.warmup
+    held = args.prompt_len + warmup + steps + decode_slack(max(batches), args.prompt_len)
+    need_tokens = max(batches) * (held + PAGE_SIZE) + PREFILL_TOKENS + 64
+    record = {"workload": "design beside its closest existing model at equal sizes", "sizes": dict(size, layers=layers),
+              "layer_runs": layer_runs, "prompt_len": args.prompt_len, "prefill_tokens": PREFILL_TOKENS, "dtype": "bf16",
+              "data": "synthetic token ids, random-init weights"}
+    for name, (cfg, vocab) in models.items():
+        rng = np.random.default_rng(0)
+        engine = Engine(config=cfg, seed=0, dtype="bfloat16", device="cuda:0", ctx=max(CONTEXT, held + 64), max_seqs=max(batches),
+                        max_batched_tokens=PREFILL_TOKENS, block_size=PAGE_SIZE, num_blocks=-(-need_tokens // PAGE_SIZE),
+                        decode_first=True, random_weights_on_device=True, ahead=not args.no_ahead)
+        out = {}
+        for batch in batches:
+            runs = [decode_run(engine, rng, vocab, batch, steps, warmup, args.prompt_len, f"{name}-b{batch}r{r}")
+                    for r in range(max(1, args.repeats))]
+            tok_s, ms, _ = median_run(runs)
+            out[f"decode_b{batch}"] = {"tokens_per_s": round(tok_s, 1), "ms_per_step": round(ms, 4)}
+            print(f"[bench] {name} decode batch {batch}: {tok_s:.1f} tok/s, {ms:.3f} ms/step", file=sys.stderr, flush=True)
+        serial = iter(range(10 ** 6))
+
+        def one_prompt():
+            engine.add_request(f"{name}-p{next(serial)}", rng.integers(0, vocab, PREFILL_TOKENS).tolist(),
+                               SamplingParams(max_tokens=1, ignore_eos=True))
+            while engine.has_unfinished():
+                engine.step()
+
+        one_prompt()
+        times = []
+        for _ in range(max(3, args.repeats)):
+            torch.cuda.synchronize()
+            start = time.perf_counter()
+            one_prompt()
+            torch.cuda.synchronize()
+            times.append(time.perf_counter() - start)
+        best = sorted(times)[len(times) // 2]
+        out["prefill"] = {"tokens_per_s": round(PREFILL_TOKENS / best, 1), "ms": round(best * 1e3, 3)}
+        print(f"[bench] {name} prefill {PREFILL_TOKENS} tokens: {best * 1e3:.2f} ms", file=sys.stderr, flush=True)
+        if not args.no_kernels:
+            out["kernels"] = {}
+            found = kernel_breakdown(one_prompt, 2, top=12)
+            if found:
+                out["kernels"]["prefill_us"] = found
+            names = [f"{name}-k{i}" for i in range(args.batch)]
+            for n in names:
+                engine.add_request(n, rng.integers(0, vocab, args.prompt_len).tolist(), SamplingParams(max_tokens=64, ignore_eos=True))
+            got = {n: 0 for n in names}
+            while min(got.values()) < 4:
+                for ev in engine.step():
+                    got[ev.request_id] += 1
+            found = kernel_breakdown(engine.step, 5, top=12)
+            if found:
+                out["kernels"][f"decode_b{args.batch}_us"] = found
+            for n in names:
+                engine.abort_request(n)
+            while engine.has_unfinished():
+                engine.step()
+            for phase, found in out["kernels"].items():
+                print(f"[bench] {name} kernels, {phase}: " + ", ".join(f"{k} {v}" for k, v in found.items()), file=sys.stderr, flush=True)
+        record[name] = out
+        del engine
+        gc.collect()
+        torch.cuda.empty_cache()
+    print(json.dumps(record), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -235,6 +344,10 @@ def main():
     ap.add_argument("--sampled", action="store_true",
                     help="for profiling the sampling kernels: the decode runs draw with temperature 0.8, top-k 50 and top-p 0.9 under a "
                          "repetition penalty of 1.1 and report 5 log-probabilities a token (the headline run is greedy)")
+    ap.add_argument("--design", choices=["menitar"], default=None,
+                    help="instead of the headline run: prefill and decode of this design beside Llama at equal sizes, with the kernels' "
+                         "device times of both; prints a line of its own")
+    ap.add_argument("--design-size", choices=sorted(DESIGN_SIZES), default="1.5b", help="with --design: the layer sizes")
     args = ap.parse_args()
     if args.gpus != 1:
         print(f"bench.py measures one GPU: this engine runs on a single MI355X, --gpus {args.gpus} is not supported")
@@ -244,6 +357,9 @@ def main():
     import torch
     from fllm_amd import Engine, SamplingParams
 
+    if args.design:
+        design_run(args)
+        return
     shape = SHAPES[args.shape]
     if args.layers is None:
         args.layers = shape["num_hidden_layers"]

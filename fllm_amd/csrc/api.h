@@ -57,6 +57,13 @@ int fllm_fused_decode_supported(int M, int K);
 // out = silu(x gate^T) * (x up^T) for bfloat16 rows x [M, K] (1..64 rows, row stride ldx; fllm_gate_up_swiglu_tiled: to 128), w = [gate; up] ([2 I, K])
 int fllm_gate_up_swiglu(const void *x, int ldx, const void *w_gate_up, const float *bias, void *out, int M, int inter,
                         int K, hipStream_t stream);
+// The gated products with the activation's constants as arguments: a(g') * (u' + offset), a(g) = g * sigmoid(alpha g),
+// g' = min(gate, limit), u' = clamp(up, -limit, limit) (limit <= 0: nothing is clamped).  fllm_norm_gate_up_glu folds the
+// RMSNorm of float32 rows in (1..64 rows); fllm_gate_up_glu takes bfloat16 rows (1..64, or 17..128 with `w_tiles`).
+int fllm_norm_gate_up_glu(const float *x, const float *norm_w, float eps, const void *w_gate_up, const float *bias, void *out,
+                          int M, int inter, int K, float limit, float alpha, float offset, hipStream_t stream);
+int fllm_gate_up_glu(const void *x, int ldx, const void *w_gate_up, const void *w_tiles, const float *bias, void *out, int M,
+                     int inter, int K, float limit, float alpha, float offset, hipStream_t stream);
 int fllm_norm_linear(const float *x, const float *norm_w, float eps, const void *w, const float *bias, void *out, int M,
                      int N, int K, hipStream_t stream);
 int fllm_norm_gate_up_swiglu(const float *x, const float *norm_w, float eps, const void *w_gate_up, const float *bias,
@@ -282,7 +289,10 @@ int fllm_talking_attention(const void *q, const void *gate, int gate_stride, con
                            const int32_t *tables, int table_stride, const int32_t *row_pos, const int32_t *row_seg,
                            const int32_t *seg_start, int num_segs, const float *talk, const float *temp, void *out, int rows,
                            int heads, int kv_heads, int k_dim, int v_dim, int page_size, float scale, int chunk, int key_chunk,
-                           int dtype, int max_context, hipStream_t stream);
+                           int dtype, int max_context, int splits, float *ws, size_t ws_floats, hipStream_t stream);
+// `splits` > 1 (bfloat16, the matrix-core kernel): that many workgroups share the keys of a tile of 16 rows and meet in
+// `ws`, float32, at least fllm_talking_attention_workspace(...) floats; the plain kernels ignore both.
+size_t fllm_talking_attention_workspace(int rows, int num_segs, int heads, int v_dim, int splits);
 
 #ifdef __cplusplus
 }

@@ -86,6 +86,9 @@ struct SkinnyArgs {
     // SCALED prologue
     const float *ssq_in;   // [M, ssq_count]
     int ssq_count;
+    // gated epilogue: g' * sigmoid(act_alpha g') * (u' + act_offset), g' = min(g, act_limit), u' = clamp(u, +-act_limit)
+    // (act_limit <= 0: nothing is clamped).  SwiGLU is alpha 1, offset 0, no limit.
+    float act_limit, act_alpha, act_offset;
 #ifdef FLLM_TIMELINE
     unsigned long long *timeline;   // measurement builds only: [workgroup][8] times of the 100 MHz clock
 #endif
@@ -218,8 +221,12 @@ __device__ __forceinline__ void epilogue(const SkinnyArgs &a, f32x4_t (&s)[RT], 
         f32x4_t act;
 #pragma unroll
         for (int i = 0; i < 4; i++) {
-            const float gt = s[0][i], up = s[RT - 1][i];
-            act[i] = gt / (1.0f + expf(-gt)) * up;
+            float gt = s[0][i], up = s[RT - 1][i];
+            if (a.act_limit > 0.f) {
+                gt = fminf(gt, a.act_limit);
+                up = fminf(fmaxf(up, -a.act_limit), a.act_limit);
+            }
+            act[i] = gt / (1.0f + expf(-(a.act_alpha * gt))) * (up + a.act_offset);
         }
         if (whole && ((uintptr_t)a.out & 7) == 0) {
             *(bf16x4_t *)((bf16_t *)a.out + (size_t)m * a.ldo + nb) = pack4(act);
@@ -1485,6 +1492,7 @@ extern "C" int fllm_norm_gate_up_swiglu(const float *x, const float *norm_w, flo
     FLLM_REQUIRE(aligned16(x) && aligned16(w_gate_up) && aligned16(norm_w), "norm_gate_up_swiglu: operands must be 16-byte aligned");
     FLLM_REQUIRE(eps > 0.f && inter > 0, "norm_gate_up_swiglu: bad eps or size");
     SkinnyArgs a = {};
+    a.act_alpha = 1.0f;      // silu(gate) * up
     a.x = x;
     a.ldx = K;
     a.norm_w = norm_w;
@@ -1507,6 +1515,7 @@ extern "C" int fllm_gate_up_swiglu(const void *x, int ldx, const void *w_gate_up
                  "gate_up_swiglu: takes 1..64 rows and K, ldx in steps of 8 (M=%d K=%d ldx=%d)", M, K, ldx);
     FLLM_REQUIRE(aligned16(x) && aligned16(w_gate_up), "gate_up_swiglu: operands must be 16-byte aligned");
     SkinnyArgs a = {};
+    a.act_alpha = 1.0f;      // silu(gate) * up
     a.x = x;
     a.ldx = ldx;
     a.w = (const bf16_t *)w_gate_up;
@@ -1617,6 +1626,7 @@ extern "C" int fllm_gate_up_swiglu_tiled(const void *x, int ldx, const void *w_g
     FLLM_REQUIRE(aligned16(x) && aligned16(w_gate_up) && (w_tiles == nullptr || aligned16(w_tiles)),
                  "gate_up_swiglu_tiled: operands must be 16-byte aligned");
     SkinnyArgs a = {};
+    a.act_alpha = 1.0f;      // silu(gate) * up
     a.x = x;
     a.ldx = ldx;
     a.w = (const bf16_t *)w_gate_up;
@@ -1724,6 +1734,7 @@ extern "C" int fllm_scaled_gate_up_swiglu(const void *xn, const float *ssq, int 
     FLLM_REQUIRE(M <= 16 || (w_tiles != nullptr && K % 256 == 0),
                  "scaled_gate_up_swiglu: from 17 rows on it takes the tile-major copy and K in steps of 256 (M=%d K=%d)", M, K);
     SkinnyArgs a = {};
+    a.act_alpha = 1.0f;      // silu(gate) * up
     a.x = xn;
     a.ldx = K;
     a.eps = eps;
@@ -1769,7 +1780,67 @@ extern "C" int fllm_scaled_qkv_rope_store(const void *xn, const float *ssq, int 
     return rc;
 }
 
-#ifdef FLLM_TIMELINE
+// The gated products with the activation's constants as arguments: out = a(g') * (u' + offset), a(g) = g * sigmoid(alpha g),
+// g' = min(x gate^T, limit), u' = clamp(x up^T, -limit, limit) (limit <= 0: nothing is clamped); w = [gate; up] ([2 I, K]).
+// fllm_norm_gate_up_glu: x is float32 [M, K] and the RMSNorm with `norm_w` is folded in (1..64 rows).
+// fllm_gate_up_glu: x is bfloat16; 1..64 rows, or 17..128 with the tile-major copy `w_tiles` (null: without).
+extern "C" int fllm_norm_gate_up_glu(const float *x, const float *norm_w, float eps, const void *w_gate_up, const float *bias, void *out,
+                                     int M, int inter, int K, float limit, float alpha, float offset, hipStream_t stream) {
+    FLLM_REQUIRE(fllm_fused_decode_supported(M, K), "norm_gate_up_glu: takes 1..64 rows and K a multiple of 8 (M=%d K=%d)", M, K);
+    FLLM_REQUIRE(aligned16(x) && aligned16(w_gate_up) && aligned16(norm_w), "norm_gate_up_glu: operands must be 16-byte aligned");
+    FLLM_REQUIRE(eps > 0.f && inter > 0, "norm_gate_up_glu: bad eps or size");
+    SkinnyArgs a = {};
+    a.act_limit = limit;
+    a.act_alpha = alpha;
+    a.act_offset = offset;
+    a.x = x;
+    a.ldx = K;
+    a.norm_w = norm_w;
+    a.eps = eps;
+    a.w = (const bf16_t *)w_gate_up;
+    a.bias = bias;
+    a.out = out;
+    a.ldo = inter;
+    a.M = M;
+    a.N = 2 * inter;
+    a.K = K;
+    const int rc = dispatch<PRO_NORM_F32, EPI_SWIGLU>(a, stream);
+    FLLM_REQUIRE(rc != 1, "norm_gate_up_glu: shape M=%d K=%d does not fit the staging area", M, K);
+    return rc;
+}
+
+extern "C" int fllm_gate_up_glu(const void *x, int ldx, const void *w_gate_up, const void *w_tiles, const float *bias, void *out, int M,
+                                int inter, int K, float limit, float alpha, float offset, hipStream_t stream) {
+    FLLM_REQUIRE(M >= 1 && M <= kWideRows && K % 8 == 0 && K >= 8 && ldx % 8 == 0 && inter > 0,
+                 "gate_up_glu: takes 1..128 rows and K, ldx in steps of 8 (M=%d K=%d ldx=%d)", M, K, ldx);
+    FLLM_REQUIRE(M <= 64 || (w_tiles != nullptr && K % 256 == 0),
+                 "gate_up_glu: beyond 64 rows it takes the tile-major copy and K in steps of 256 (M=%d K=%d)", M, K);
+    FLLM_REQUIRE(aligned16(x) && aligned16(w_gate_up) && (w_tiles == nullptr || aligned16(w_tiles)),
+                 "gate_up_glu: operands must be 16-byte aligned");
+    SkinnyArgs a = {};
+    a.act_limit = limit;
+    a.act_alpha = alpha;
+    a.act_offset = offset;
+    a.x = x;
+    a.ldx = ldx;
+    a.w = (const bf16_t *)w_gate_up;
+    a.bias = bias;
+    a.out = out;
+    a.ldo = inter;
+    a.M = M;
+    a.N = 2 * inter;
+    a.K = K;
+    if (M >= 17 && w_tiles != nullptr) {
+        a.w_tiles = (const bf16_t *)w_tiles;
+        return dispatch_wide<EPI_SWIGLU>(a, stream);
+    }
+    const int rc = dispatch<PRO_BF16, EPI_SWIGLU>(a, stream);
+    FLLM_REQUIRE(rc != 1, "gate_up_glu: shape M=%d K=%d does not fit", M, K);
+    return rc;
+}
+
+
 // measurement builds only: device memory for [workgroups][8] clock readings of the next resident launches (null: off)
+#ifdef FLLM_TIMELINE
 extern "C" void fllm_set_timeline(unsigned long long *buffer) { g_timeline = buffer; }
 #endif

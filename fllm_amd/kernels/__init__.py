@@ -87,6 +87,9 @@ def load_library(build_if_missing: bool = True):
                                   c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void, c_void],
         "fllm_norm_linear": [c_void, c_void, c_float, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
         "fllm_norm_gate_up_swiglu": [c_void, c_void, c_float, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
+        "fllm_norm_gate_up_glu": [c_void, c_void, c_float, c_void, c_void, c_void, c_int, c_int, c_int, c_float, c_float, c_float,
+                                  c_void],
+        "fllm_gate_up_glu": [c_void, c_int, c_void, c_void, c_void, c_void, c_int, c_int, c_int, c_float, c_float, c_float, c_void],
         "fllm_norm_qkv_rope_store": [c_void, c_void, c_float, c_void, c_void, c_void, c_void, c_void, c_void, c_int, c_void,
                                      c_void, c_int, c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void],
         "fllm_argmax": [c_void, c_void, c_int, c_int, c_void],
@@ -115,7 +118,7 @@ def load_library(build_if_missing: bool = True):
                                     c_void],
         "fllm_talking_attention": [c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_void,
                                    c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int,
-                                   c_void],
+                                   c_int, c_void, ctypes.c_size_t, c_void],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)
@@ -541,6 +544,38 @@ class Ops:
                                                  two_i // 2, K, self._stream()))
         return out
 
+    def norm_gate_up_glu(self, x, norm_weight, eps, w_gate_up, out, limit: float, alpha: float, up_offset: float, bias=None):
+        """`norm_gate_up_swiglu` with the activation's constants as arguments: out = a(g') * (u' + up_offset) with
+        a(g) = g * sigmoid(alpha * g), g' = min(gate, limit), u' = clamp(up, -limit, limit) (limit <= 0: nothing is
+        clamped), gate and up the two halves of rmsnorm(x) @ w_gate_up.T; x float32 [M <= 64, K], out bfloat16 [M, I]."""
+        two_i = w_gate_up.shape[0]
+        _need(two_i % 2 == 0, "w_gate_up needs an even number of rows")
+        M, K = self._fused_operands(x, norm_weight, w_gate_up, bias, two_i)
+        _dense(out, "out", torch.bfloat16, (M, two_i // 2))
+        self._check(self.lib.fllm_norm_gate_up_glu(_ptr(x), _ptr(norm_weight), float(eps), _ptr(w_gate_up), _ptr(bias), _ptr(out), M,
+                                                   two_i // 2, K, float(limit), float(alpha), float(up_offset), self._stream()))
+        return out
+
+    def gate_up_glu(self, x, w_gate_up, out, limit: float, alpha: float, up_offset: float, bias=None):
+        """`gate_up_swiglu` with the activation's constants as arguments (see `norm_gate_up_glu`): up to 64 bfloat16 rows,
+        up to 128 with the tile-major copy of w_gate_up."""
+        M, K = x.shape
+        two_i = w_gate_up.shape[0]
+        _need(two_i % 2 == 0, "w_gate_up needs an even number of rows")
+        _need(x.dtype == torch.bfloat16 and x.is_cuda and x.stride(1) == 1, "x must be bfloat16 rows on the GPU")
+        _need(M == 1 or x.stride(0) % 8 == 0, "rows of x must begin on 16 bytes")
+        _dense(w_gate_up, "w_gate_up", torch.bfloat16, (two_i, K))
+        if bias is not None:
+            _dense(bias, "bias", torch.float32, (two_i,))
+        _dense(out, "out", torch.bfloat16, (M, two_i // 2))
+        _need(1 <= M <= self.GATE_UP_SWIGLU_TILED_ROWS and K % 8 == 0, f"gate_up_glu takes 1..128 rows and widths in steps of 8, not {M} x {K}")
+        tiles = self._tiles_of(w_gate_up, gate_up=True) if M >= 17 and Ops._tiles else None
+        _need(M <= 64 or (tiles is not None and K % 256 == 0),
+              f"gate_up_glu takes more than 64 rows only with the tile-major copy of the matrix and widths in steps of 256, not {M} x {K}")
+        self._check(self.lib.fllm_gate_up_glu(_ptr(x), x.stride(0) if M > 1 else K, _ptr(w_gate_up), _ptr(tiles), _ptr(bias), _ptr(out),
+                                              M, two_i // 2, K, float(limit), float(alpha), float(up_offset), self._stream()))
+        return out
+
     def norm_qkv_rope_store(self, x, norm_weight, eps, w_qkv, q_out, row_pos, row_seg, tables, cos, sin, k_pages, v_pages,
                             heads, kv_heads, head_dim, rope_dims, page_size, bias=None, prepared: Optional[PreparedNorm] = None):
         """q, k, v = rmsnorm(x) @ w_qkv.T; rotary on pairs (2l, 2l+1) of q and k; q to `q_out`
@@ -761,10 +796,29 @@ class Ops:
             k_dim, v_dim, rope_dims, page_size, key_chunk, _DTYPE_CODE[qkv.dtype], 1 if store else 0, self._stream()))
         return q_out
 
+    TALKING_TILE_ROWS = 16          # rows of one request that a workgroup of the matrix-core kernel takes
+    TALKING_KEY_BLOCK = 64          # keys it walks at a time
+    TALKING_WORKGROUPS = 512        # what a launch should come to: two a compute unit
+
+    def talking_attention_splits(self, rows: int, num_segs: int, chunk: Optional[int], max_context: int) -> int:
+        """How many workgroups should share the keys of a row tile of `talking_attention` (1: none): enough to fill the
+        device when the step has few tiles (a decode step has one a request), at most one a block of keys."""
+        tiles = rows // self.TALKING_TILE_ROWS + num_segs
+        span = max_context if not chunk else min(max_context, chunk + self.TALKING_TILE_ROWS)
+        blocks = -(-(span + self.TALKING_TILE_ROWS) // self.TALKING_KEY_BLOCK)
+        return max(1, min(self.TALKING_WORKGROUPS // max(tiles, 1), blocks, 64))
+
+    def talking_attention_workspace(self, rows: int, num_segs: int, heads: int, v_dim: int, splits: int) -> int:
+        """float32 elements of workspace that `splits` workgroups a tile need."""
+        if splits <= 1:
+            return 0
+        return (rows // self.TALKING_TILE_ROWS + num_segs) * splits * self.TALKING_TILE_ROWS * heads * (2 + v_dim)
+
     def talking_attention(self, q: torch.Tensor, gate: Optional[torch.Tensor], k_pages: torch.Tensor, v_pages: torch.Tensor,
                           tables: torch.Tensor, row_pos: torch.Tensor, row_seg: torch.Tensor, seg_start: torch.Tensor,
                           talk: torch.Tensor, temp: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int, k_dim: int,
-                          v_dim: int, page_size: int, scale: float, chunk: Optional[int], key_chunk: int, max_context: int) -> torch.Tensor:
+                          v_dim: int, page_size: int, scale: float, chunk: Optional[int], key_chunk: int, max_context: int,
+                          splits: int = 1, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
         """Attention whose scores are mixed across heads before the softmax (score[h] = sum_g talk[h, g] * q_g . k * scale *
         temp[g]) over the keys of the row's own chunk of `chunk` positions up to the row (None: all keys up to the row);
         head h's output times sigmoid(gate[row, h]) (`gate` may be a column slice of a wider matrix; None: no gate)."""
@@ -786,11 +840,16 @@ class Ops:
         _dense(talk, "talk", torch.float32, (heads, heads))
         _dense(temp, "temp", torch.float32, (heads,))
         _dense(out, "out", q.dtype, (rows, heads * v_dim))
+        ws_floats = 0
+        if splits > 1:
+            _need(workspace is not None, "workgroups that share a tile need a workspace")
+            _dense(workspace, "workspace", torch.float32)
+            ws_floats = workspace.numel()
         self._check(self.lib.fllm_talking_attention(
             _ptr(q), _ptr(gate), gate_stride, _ptr(k_pages), _ptr(v_pages), _ptr(tables), tables.shape[1], _ptr(row_pos),
             _ptr(row_seg), _ptr(seg_start), seg_start.numel() - 1, _ptr(talk), _ptr(temp), _ptr(out), rows, heads, kv_heads, k_dim,
             v_dim, page_size, float(scale), int(chunk) if chunk else 0, key_chunk, _DTYPE_CODE[q.dtype], int(max_context),
-            self._stream()))
+            int(splits), _ptr(workspace), ws_floats, self._stream()))
         return out
 
     def measured_ceilings(self, read_bytes: int = 4 << 30, repeats: int = 5) -> dict:

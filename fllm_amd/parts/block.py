@@ -101,21 +101,38 @@ class ParallelBlock(Block):
     def forward(self, ctx, residual, binding):
         rt, ops = self.rt, self.rt.ops
         ctx.then_norm = ctx.prepared = None          # the sums of this block's parts are not read by a norm they know
-        first = getattr(self.mixer_norm, "fused_prologue", lambda: None)()
-        second = getattr(self.feed_forward_norm, "fused_prologue", lambda: None)() if self.feed_forward is not None else None
-        pair = getattr(ops, "rmsnorm_pair", None)
+        # a part may read the stream through its norm in one kernel with its first product, and add to it later: every
+        # reader of the stream runs before the first sum into it
+        project = getattr(self.mixer, "project_from_residual", None)
+        projected = project(ctx, residual, self.mixer_norm) if project is not None else None
         if self.feed_forward is None:
-            self.mixer.forward(ctx, self.mixer_norm.forward(ctx, residual), residual, binding)
+            if projected is not None:
+                self.mixer.attend(ctx, projected, residual, binding)
+            else:
+                self.mixer.forward(ctx, self.mixer_norm.forward(ctx, residual), residual, binding)
             return
-        if pair is not None and first is not None and second is not None:
-            h_mixer, h_ff = rt.empty(tuple(residual.shape)), rt.empty(tuple(residual.shape))
-            pair(residual, first[0], first[1], h_mixer, second[0], second[1], h_ff)
-        else:
+        begin = getattr(self.feed_forward, "begin_from_residual", None)
+        begun = begin(ctx, residual, self.feed_forward_norm) if begin is not None else None
+        h_mixer = h_ff = None
+        if projected is None and begun is None:
+            first = getattr(self.mixer_norm, "fused_prologue", lambda: None)()
+            second = getattr(self.feed_forward_norm, "fused_prologue", lambda: None)()
+            pair = getattr(ops, "rmsnorm_pair", None)
+            if pair is not None and first is not None and second is not None:
+                h_mixer, h_ff = rt.empty(tuple(residual.shape)), rt.empty(tuple(residual.shape))
+                pair(residual, first[0], first[1], h_mixer, second[0], second[1], h_ff)
+        if projected is None and h_mixer is None:
             h_mixer = self.mixer_norm.forward(ctx, residual)
+        if begun is None and h_ff is None:
             h_ff = self.feed_forward_norm.forward(ctx, residual)
-        # both inputs exist before either branch adds to the stream
-        self.mixer.forward(ctx, h_mixer, residual, binding)
-        self.feed_forward.forward(ctx, h_ff, residual)
+        if projected is not None:
+            self.mixer.attend(ctx, projected, residual, binding)
+        else:
+            self.mixer.forward(ctx, h_mixer, residual, binding)
+        if begun is not None:
+            self.feed_forward.finish(ctx, begun, residual)
+        else:
+            self.feed_forward.forward(ctx, h_ff, residual)
 
 
 register_part("block", "prenorm", PreNormBlock)

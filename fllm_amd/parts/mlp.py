@@ -123,14 +123,41 @@ class ClampedGLU(FeedForward):
         self.w_gate_up = torch.cat([rt.matrix(weights["gate"]), rt.matrix(weights["up"])], dim=0).contiguous()
         self.w_down = rt.matrix(weights["down"])
         rt.tile_for_decode(self.w_down)
+        rt.tile_for_decode(self.w_gate_up, gate_up=True, priority=1)
+
+    def begin_from_residual(self, ctx, residual, norm):
+        """Decode-sized steps in bfloat16: the norm before this part, the gate/up product and the activation are one
+        kernel that reads the residual stream; the activations come back and `finish` adds the down projection, which
+        lets an arrangement run other readers of the same stream in between.  None: not taken."""
+        rt, ops = self.rt, self.rt.ops
+        rows = residual.shape[0]
+        prologue = getattr(norm, "fused_prologue", lambda: None)()
+        if rt.dtype != torch.bfloat16 or prologue is None or not hasattr(ops, "norm_gate_up_glu"):
+            return None
+        if fused_form(ops, rows, self.hidden, self.w_gate_up, gate_up=True) != "resident":
+            return None
+        act = rt.empty((rows, self.inter))
+        ops.norm_gate_up_glu(residual, prologue[0], prologue[1], self.w_gate_up, act, self.limit, self.alpha, self.up_offset)
+        return act
+
+    def finish(self, ctx, act, residual):
+        self.rt.ops.linear(act, self.w_down, residual, accumulate=True)
 
     def forward(self, ctx, h, residual):
         rt, ops = self.rt, self.rt.ops
         rows = h.shape[0]
-        gate_up = rt.empty((rows, 2 * self.inter))
-        ops.linear(h, self.w_gate_up, gate_up)
         act = rt.empty((rows, self.inter))
-        ops.glu_clamped(gate_up, act, self.limit, self.alpha, self.up_offset)
+        start = getattr(ops, "library_gemm_from", None)
+        own = getattr(ops, "own_feed_forward", None)
+        if (rt.dtype == torch.bfloat16 and hasattr(ops, "gate_up_glu") and self.hidden % 8 == 0 and h.stride(0) % 8 == 0
+                and ((own is not None and own(rows, self.w_gate_up, self.w_down))
+                     or (rows <= getattr(ops, "GATE_UP_SWIGLU_ROWS", 0) and (start is None or rows < start)))):
+            # steps that the hand-written products serve: the activation is the epilogue of the gate/up product
+            ops.gate_up_glu(h, self.w_gate_up, act, self.limit, self.alpha, self.up_offset)
+        else:
+            gate_up = rt.empty((rows, 2 * self.inter))
+            ops.linear(h, self.w_gate_up, gate_up)
+            ops.glu_clamped(gate_up, act, self.limit, self.alpha, self.up_offset)
         ops.linear(act, self.w_down, residual, accumulate=True)
 
 

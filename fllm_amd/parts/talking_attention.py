@@ -14,7 +14,7 @@ import torch
 
 from ..config.spec import PartSpec
 from ..registry import part_class, register_part
-from .base import INIT_MATRIX, INIT_NORM, KVNeed, Mixer
+from .base import INIT_MATRIX, INIT_NORM, KVNeed, Mixer, fused_form
 
 
 class TalkingAttention(Mixer):
@@ -68,6 +68,7 @@ class TalkingAttention(Mixer):
         self.gate_at = self.heads * self.k_dim + self.kv_heads * (self.k_dim + self.v_dim)
         self.w_o = rt.matrix(weights["o"])
         rt.tile_for_decode(self.w_o)
+        rt.tile_for_decode(self.w_qkvg, priority=1)
         self.q_norm = rt.vector(weights["q_norm"])
         self.k_norm = rt.vector(weights["k_norm"])
         self.talk = rt.vector(weights["talk"])
@@ -78,12 +79,30 @@ class TalkingAttention(Mixer):
         # the request until it ends
         return KVNeed(self.kv_heads, self.k_dim, self.v_dim, None, key_chunk=self.key_chunk)
 
-    def forward(self, ctx, h, residual, binding):
+    def project_from_residual(self, ctx, residual, norm):
+        """Decode-sized steps in bfloat16: the norm before the mixer and the joint product are one kernel that reads the
+        residual stream; `attend` goes on from the product.  None: not taken."""
         rt, ops = self.rt, self.rt.ops
-        rows = h.shape[0]
-        nh, nkv, d, dv = self.heads, self.kv_heads, self.k_dim, self.v_dim
+        rows = residual.shape[0]
+        prologue = getattr(norm, "fused_prologue", lambda: None)()
+        if rt.dtype != torch.bfloat16 or prologue is None or not hasattr(ops, "norm_linear"):
+            return None
+        if fused_form(ops, rows, self.hidden, self.w_qkvg) != "resident":
+            return None
         qkvg = rt.empty((rows, self.w_qkvg.shape[0]))
-        ops.linear(h, self.w_qkvg, qkvg)
+        ops.norm_linear(residual, prologue[0], prologue[1], self.w_qkvg, qkvg)
+        return qkvg
+
+    def forward(self, ctx, h, residual, binding):
+        qkvg = self.rt.empty((h.shape[0], self.w_qkvg.shape[0]))
+        self.rt.ops.linear(h, self.w_qkvg, qkvg)
+        self.attend(ctx, qkvg, residual, binding)
+
+    def attend(self, ctx, qkvg, residual, binding):
+        """From the joint product [q | k | v | gate] of the step's rows to the sum into the residual stream."""
+        rt, ops = self.rt, self.rt.ops
+        rows = qkvg.shape[0]
+        nh, nkv, d, dv = self.heads, self.kv_heads, self.k_dim, self.v_dim
         tables = ctx.tables[binding.group]
         if self.position is not None:
             cos, sin, dims = self.position.cos, self.position.sin, self.position.dims
@@ -94,9 +113,18 @@ class TalkingAttention(Mixer):
                                binding.k_pages if binding.writes else None, binding.v_pages if binding.writes else None,
                                nh, nkv, d, dv, dims, binding.page_size, self.key_chunk)
         out = rt.empty((rows, nh * dv))
+        # few row tiles (a decode step has one a request): several workgroups share a tile's keys and meet in a workspace
+        extra = {}
+        split = getattr(ops, "talking_attention_splits", None)
+        if split is not None and rt.dtype == torch.bfloat16:
+            segments = ctx.seg_start.numel() - 1
+            splits = split(rows, segments, self.chunk, ctx.max_context)
+            if splits > 1:
+                extra = {"splits": splits, "workspace": rt.empty((ops.talking_attention_workspace(rows, segments, nh, dv, splits),),
+                                                                 dtype=torch.float32)}
         ops.talking_attention(q, qkvg[:, self.gate_at:self.gate_at + nh], binding.k_pages, binding.v_pages, tables,
                               ctx.row_pos, ctx.row_seg, ctx.seg_start, self.talk, self.temp, out, nh, nkv, d, dv,
-                              binding.page_size, self.scale, self.chunk, self.key_chunk, ctx.max_context)
+                              binding.page_size, self.scale, self.chunk, self.key_chunk, ctx.max_context, **extra)
         ops.linear(out, self.w_o, residual, accumulate=True)
 
 

@@ -8,7 +8,7 @@ import numpy as np
 import torch
 
 
-def layer(heads, kv_heads, dim, vdim, chunk=None, rot=None, ff=None, limit=1.5, scale=None):
+def layer(heads, kv_heads, dim, vdim, chunk=None, rot=None, ff=None, limit=2.0, scale=None):
     mixer = {"heads": heads, "kv_heads": kv_heads, "dim": dim, "vdim": vdim, "scale": scale if scale is not None else dim ** -0.5}
     if chunk is not None:
         mixer["mask"] = {"size": chunk}
@@ -37,9 +37,9 @@ Q = config(96, 120, [layer(3, 3, 32, 32, chunk=40, rot=(32, 500.0), ff=112),
 # (every earlier key is seen), a loop of one pass over the last layer
 R = config(48, 80, [layer(2, 1, 20, 12, ff=64), layer(2, 1, 20, 12, ff=64, limit=3.0)], loop=(1, 2, 1), embedding_scale=1.0)
 # S: layers of different geometry (two cache groups), sizes the matrix-core kernel takes, a loop in the middle
-S = config(128, 160, [layer(8, 2, 64, 32, chunk=80, rot=(32, 20000.0), ff=192),
+S = config(128, 160, [layer(8, 2, 64, 32, chunk=80, rot=(32, 25000.0), ff=192),
                       layer(2, 1, 32, 64, chunk=16, rot=(8, 100.0), ff=192),
-                      layer(8, 2, 64, 32, chunk=80, rot=(32, 20000.0), ff=192)], loop=(1, 3, 2))
+                      layer(8, 2, 64, 32, chunk=80, rot=(32, 25000.0), ff=192)], loop=(1, 3, 2))
 # T: twelve heads (the wider instance of the matrix-core kernel), a chunk of one page
 T = config(64, 72, [layer(12, 4, 32, 16, chunk=16, rot=(32, 3000.0), ff=96)])
 CONFIGS = {"P": P, "Q": Q, "R": R, "S": S, "T": T}

@@ -61,7 +61,7 @@ def test_two_norms_of_one_row(ops, ref, rows, width, out_dtype):
 
 
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
-@pytest.mark.parametrize("limit,alpha,offset", [(1.5, 1.702, 1.0), (0.5, 1.0, 0.0), (0.0, 1.702, 1.0)])
+@pytest.mark.parametrize("limit,alpha,offset", [(1.25, 1.702, 1.0), (0.5, 1.0, 0.0), (0.0, 1.702, 1.0)])
 @pytest.mark.parametrize("rows,inter", [(1, 24), (9, 333), (70, 2048)])
 def test_clamped_gated_activation(ops, ref, rows, inter, limit, alpha, offset, dtype):
     gate_up = (torch.randn(rows, 2 * inter, generator=gen(4)) * 2).to(dtype)      # many values beyond either limit
@@ -89,6 +89,60 @@ def test_what_a_pass_adds_to_the_stream(ops, ref, table_dtype):
     y = x.to(DEV).clone()
     ops.scale_(y, 0.37)
     close(y, x.double() * 0.37, 1e-6, 0, "scale")
+
+
+@pytest.mark.parametrize("rows", [1, 8, 16, 33, 64])
+@pytest.mark.parametrize("limit,alpha,offset", [(1.25, 1.702, 1.0), (0.0, 1.0, 0.0)])
+def test_gated_products_with_the_activation_as_their_epilogue(ops, ref, rows, limit, alpha, offset):
+    """The decode forms: norm, gate/up product and clamped activation in one kernel from the float32 stream, and the
+    product with the activation from bfloat16 rows, against norm, product and activation done apart in float64."""
+    K, inter = 192, 328
+    x = torch.randn(rows, K, generator=gen(11)) * 2
+    norm_w = 1 + 0.3 * torch.randn(K, generator=gen(12))
+    w = (torch.randn(2 * inter, K, generator=gen(13)) * (3.0 / K ** 0.5)).to(torch.bfloat16)      # many products beyond the limit
+    h = torch.empty(rows, K, dtype=torch.float64)
+    ref.rmsnorm(x.double(), norm_w, 1e-5, h)
+    want = torch.empty(rows, inter, dtype=torch.float64)
+    ref.glu_clamped(h @ w.double().T, want, limit, alpha, offset)
+    # the fused kernel multiplies the row by the norm's weight, rounds that to bfloat16 for the matrix cores and scales the
+    # sums by the row's 1 / rms afterwards: the reference rounds at the same place, the rest in float64
+    xw = (x * norm_w).to(torch.bfloat16).double()
+    inv = 1.0 / torch.sqrt((x.double() ** 2).mean(-1, keepdim=True) + 1e-5)
+    want_f = torch.empty(rows, inter, dtype=torch.float64)
+    ref.glu_clamped((xw @ w.double().T) * inv, want_f, limit, alpha, offset)
+    got = torch.empty(rows, inter, dtype=torch.bfloat16, device=DEV)
+    ops.norm_gate_up_glu(x.to(DEV), norm_w.to(DEV), 1e-5, w.to(DEV), got, limit, alpha, offset)
+    close(got, want_f, 2 * BF16_EPS, 1e-2, "norm + product + activation")
+    assert (got.double().cpu() - want).abs().max() <= 0.02 * want.abs().max()        # and near the unrounded order
+    hb = h.to(torch.bfloat16)
+    want_b = torch.empty(rows, inter, dtype=torch.float64)
+    ref.glu_clamped(hb.double() @ w.double().T, want_b, limit, alpha, offset)
+    got = torch.empty(rows, inter, dtype=torch.bfloat16, device=DEV)
+    ops.gate_up_glu(hb.to(DEV), w.to(DEV), got, limit, alpha, offset)
+    close(got, want_b, 2 * BF16_EPS, 1e-2, "product + activation")
+    if limit == 0.0:        # the constants of SwiGLU give SwiGLU's own kernel bit for bit
+        same = torch.empty_like(got)
+        ops.gate_up_swiglu(hb.to(DEV), w.to(DEV), same)
+        assert torch.equal(got, same)
+
+
+def test_decode_steps_take_the_fused_forms(models, monkeypatch):
+    """A bfloat16 decode step reads the stream through both norms inside the products' kernels: no norm kernel and no
+    activation kernel of their own run."""
+    from fllm_amd.engine import StepEntry
+    from fllm_amd.kernels import Ops
+    folder, cfg, requests, _, _ = models["S"]
+    runner = make_runner(folder, "bfloat16", 16, 256, use_graphs=False)
+    calls = []
+    for name in ("rmsnorm_pair", "glu_clamped", "norm_linear", "norm_gate_up_glu", "gate_up_glu"):
+        inner = getattr(Ops, name)
+        monkeypatch.setattr(Ops, name, lambda self, *a, _n=name, _i=inner, **k: (calls.append(_n), _i(self, *a, **k))[1])
+    toks = requests["r0"]
+    runner.step([StepEntry("a", toks[:40], [])])
+    assert "norm_linear" not in calls and "norm_gate_up_glu" not in calls and "rmsnorm_pair" in calls
+    calls.clear()
+    runner.step([StepEntry("a", toks[40:41], [0])])
+    assert set(calls) == {"norm_linear", "norm_gate_up_glu"}, calls
 
 
 # ---------------------------------------------------------------------------------------------
@@ -144,7 +198,7 @@ class Scene:
         return out
 
 
-def run_mixer_kernels(o, t, sc, chunk, scale, dtype):
+def run_mixer_kernels(o, t, sc, chunk, scale, dtype, splits=1):
     rows = t["qkvg"].shape[0]
     H, G, d, dv = sc.H, sc.G, sc.d, sc.dv
     q = torch.empty(rows, H * d, dtype=dtype, device=t["qkvg"].device)
@@ -152,8 +206,13 @@ def run_mixer_kernels(o, t, sc, chunk, scale, dtype):
                          t["sin"], t["k_pages"], t["v_pages"], H, G, d, dv, sc.rope_dims, sc.page, sc.key_chunk)
     out = torch.empty(rows, H * dv, dtype=dtype, device=q.device)
     gate_at = H * d + G * (d + dv)
+    extra = {}
+    if splits > 1:      # several workgroups share a row tile's keys and meet in a workspace
+        segments = t["seg_start"].numel() - 1
+        extra = {"splits": splits, "workspace": torch.empty(o.talking_attention_workspace(rows, segments, H, dv, splits),
+                                                            dtype=torch.float32, device=q.device)}
     o.talking_attention(q, t["qkvg"][:, gate_at:gate_at + H], t["k_pages"], t["v_pages"], t["tables"], t["row_pos"], t["row_seg"],
-                        t["seg_start"], t["talk"], t["temp"], out, H, G, d, dv, sc.page, scale, chunk, sc.key_chunk, sc.max_pos)
+                        t["seg_start"], t["talk"], t["temp"], out, H, G, d, dv, sc.page, scale, chunk, sc.key_chunk, sc.max_pos, **extra)
     return q, out
 
 
@@ -166,12 +225,13 @@ SHAPES = [(4, 2, 32, 16, 24, 8, 16), (6, 3, 64, 64, 40, 16, 32), (12, 4, 32, 16,
 SEGMENTS = [(0, 50), (37, 1), (23, 30), (79, 2), (80, 1), (95, 18), (0, 1), (120, 1), (47, 1), (48, 1), (2, 2), (199, 1)]
 
 
-@pytest.mark.parametrize("fast", [True, False])
+@pytest.mark.parametrize("fast", [True, False, 2, 5])      # a number: the matrix-core kernel with that many workgroups a row tile
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("shape", SHAPES)
 def test_mixed_head_attention_over_pages(ops, ref, shape, dtype, fast):
     H, G, d, dv, chunk, page, rope_dims = shape
-    if dtype == torch.float32 and not fast:
+    splits, fast = (fast, True) if fast not in (True, False) else (1, fast)
+    if dtype == torch.float32 and (not fast or splits > 1):
         pytest.skip("float32 has one kernel")
     scale = d ** -0.5 * 1.3
     # loud keys at the edges of what a row may see: the last position of the chunk before its own, and the position after
@@ -188,7 +248,7 @@ def test_mixed_head_attention_over_pages(ops, ref, shape, dtype, fast):
     ops.set_fast_kernels(fast)
     try:
         got_t = sc.tensors(DEV)
-        got_q, got = run_mixer_kernels(ops, got_t, sc, chunk, scale, dtype)
+        got_q, got = run_mixer_kernels(ops, got_t, sc, chunk, scale, dtype, splits)
         torch.cuda.synchronize()
     finally:
         ops.set_fast_kernels(True)

@@ -289,9 +289,10 @@ int fllm_talking_attention(const void *q, const void *gate, int gate_stride, con
                            const int32_t *tables, int table_stride, const int32_t *row_pos, const int32_t *row_seg,
                            const int32_t *seg_start, int num_segs, const float *talk, const float *temp, void *out, int rows,
                            int heads, int kv_heads, int k_dim, int v_dim, int page_size, float scale, int chunk, int key_chunk,
-                           int dtype, int max_context, int splits, float *ws, size_t ws_floats, hipStream_t stream);
+                           int dtype, int max_context, int splits, float *ws, size_t ws_floats, int single_rows, hipStream_t stream);
 // `splits` > 1 (bfloat16, the matrix-core kernel): that many workgroups share the keys of a tile of 16 rows and meet in
-// `ws`, float32, at least fllm_talking_attention_workspace(...) floats; the plain kernels ignore both.
+// `ws`, float32, at least fllm_talking_attention_workspace(...) floats; the plain kernels ignore both.  `single_rows`: the
+// caller knows that every segment has one row (a decode step), which has a matrix-core kernel of its own.
 size_t fllm_talking_attention_workspace(int rows, int num_segs, int heads, int v_dim, int splits);
 
 #ifdef __cplusplus

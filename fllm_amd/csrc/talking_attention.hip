@@ -20,7 +20,7 @@ int fllm_talking_attention_bf16_fast(const void *q, const void *gate, int gate_s
                                      const int32_t *tables, int table_stride, const int32_t *row_pos, const int32_t *row_seg,
                                      const int32_t *seg_start, int num_segs, const float *talk, const float *temp, void *out,
                                      int rows, int heads, int kv_heads, int k_dim, int v_dim, int page_size, float scale, int chunk,
-                                     int key_chunk, int max_context, int splits, float *ws, size_t ws_floats,
+                                     int key_chunk, int max_context, int splits, float *ws, size_t ws_floats, int single_rows,
                                      hipStream_t stream);   // talking_attention_mfma.hip; 1: declined
 
 namespace {
@@ -232,7 +232,7 @@ extern "C" int fllm_talking_attention(const void *q, const void *gate, int gate_
                                       const int32_t *seg_start, int num_segs, const float *talk, const float *temp, void *out,
                                       int rows, int heads, int kv_heads, int k_dim, int v_dim, int page_size, float scale,
                                       int chunk, int key_chunk, int dtype, int max_context, int splits, float *ws, size_t ws_floats,
-                                      hipStream_t stream) {
+                                      int single_rows, hipStream_t stream) {
     FLLM_REQUIRE(rows >= 0 && heads > 0 && kv_heads > 0 && k_dim > 0 && v_dim > 0 && page_size > 0 && table_stride > 0,
                  "talking_attention: bad sizes");
     FLLM_REQUIRE(heads % kv_heads == 0, "talking_attention: %d heads are not a multiple of %d key/value heads", heads, kv_heads);
@@ -244,7 +244,7 @@ extern "C" int fllm_talking_attention(const void *q, const void *gate, int gate_
     if (dtype == FLLM_BF16 && fllm_fast_kernels_enabled()) {
         const int fast = fllm_talking_attention_bf16_fast(q, gate, gate_stride, k_pages, v_pages, tables, table_stride, row_pos, row_seg,
                                                           seg_start, num_segs, talk, temp, out, rows, heads, kv_heads, k_dim, v_dim,
-                                                          page_size, scale, chunk, key_chunk, max_context, splits, ws, ws_floats, stream);
+                                                          page_size, scale, chunk, key_chunk, max_context, splits, ws, ws_floats, single_rows, stream);
         if (fast <= 0) return fast;
     }
     FLLM_REQUIRE(heads * v_dim <= kBlock * kMaxOut, "talking_attention: %d heads of %d values are more than %d outputs a row", heads,

@@ -118,7 +118,7 @@ def load_library(build_if_missing: bool = True):
                                     c_void],
         "fllm_talking_attention": [c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_void,
                                    c_void, c_void, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int,
-                                   c_int, c_void, ctypes.c_size_t, c_void],
+                                   c_int, c_void, ctypes.c_size_t, c_int, c_void],
     }
     for name, args in sig.items():
         fn = getattr(lib, name)
@@ -818,7 +818,7 @@ class Ops:
                           tables: torch.Tensor, row_pos: torch.Tensor, row_seg: torch.Tensor, seg_start: torch.Tensor,
                           talk: torch.Tensor, temp: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int, k_dim: int,
                           v_dim: int, page_size: int, scale: float, chunk: Optional[int], key_chunk: int, max_context: int,
-                          splits: int = 1, workspace: Optional[torch.Tensor] = None) -> torch.Tensor:
+                          splits: int = 1, workspace: Optional[torch.Tensor] = None, single_rows: bool = False) -> torch.Tensor:
         """Attention whose scores are mixed across heads before the softmax (score[h] = sum_g talk[h, g] * q_g . k * scale *
         temp[g]) over the keys of the row's own chunk of `chunk` positions up to the row (None: all keys up to the row);
         head h's output times sigmoid(gate[row, h]) (`gate` may be a column slice of a wider matrix; None: no gate)."""
@@ -849,7 +849,7 @@ class Ops:
             _ptr(q), _ptr(gate), gate_stride, _ptr(k_pages), _ptr(v_pages), _ptr(tables), tables.shape[1], _ptr(row_pos),
             _ptr(row_seg), _ptr(seg_start), seg_start.numel() - 1, _ptr(talk), _ptr(temp), _ptr(out), rows, heads, kv_heads, k_dim,
             v_dim, page_size, float(scale), int(chunk) if chunk else 0, key_chunk, _DTYPE_CODE[q.dtype], int(max_context),
-            int(splits), _ptr(workspace), ws_floats, self._stream()))
+            int(splits), _ptr(workspace), ws_floats, 1 if single_rows and rows == seg_start.numel() - 1 else 0, self._stream()))
         return out
 
     def measured_ceilings(self, read_bytes: int = 4 << 30, repeats: int = 5) -> dict:

@@ -114,13 +114,13 @@ class TalkingAttention(Mixer):
                                nh, nkv, d, dv, dims, binding.page_size, self.key_chunk)
         out = rt.empty((rows, nh * dv))
         # few row tiles (a decode step has one a request): several workgroups share a tile's keys and meet in a workspace
-        extra = {}
+        extra = {"single_rows": True} if getattr(ctx, "uniform_rows", False) and hasattr(ops, "talking_attention_splits") else {}
         split = getattr(ops, "talking_attention_splits", None)
         if split is not None and rt.dtype == torch.bfloat16:
             segments = ctx.seg_start.numel() - 1
             splits = split(rows, segments, self.chunk, ctx.max_context)
             if splits > 1:
-                extra = {"splits": splits, "workspace": rt.empty((ops.talking_attention_workspace(rows, segments, nh, dv, splits),),
+                extra = {**extra, "splits": splits, "workspace": rt.empty((ops.talking_attention_workspace(rows, segments, nh, dv, splits),),
                                                                  dtype=torch.float32)}
         ops.talking_attention(q, qkvg[:, self.gate_at:self.gate_at + nh], binding.k_pages, binding.v_pages, tables,
                               ctx.row_pos, ctx.row_seg, ctx.seg_start, self.talk, self.temp, out, nh, nkv, d, dv,

@@ -198,7 +198,7 @@ class Scene:
         return out
 
 
-def run_mixer_kernels(o, t, sc, chunk, scale, dtype, splits=1):
+def run_mixer_kernels(o, t, sc, chunk, scale, dtype, splits=1, single_rows=False):
     rows = t["qkvg"].shape[0]
     H, G, d, dv = sc.H, sc.G, sc.d, sc.dv
     q = torch.empty(rows, H * d, dtype=dtype, device=t["qkvg"].device)
@@ -206,10 +206,10 @@ def run_mixer_kernels(o, t, sc, chunk, scale, dtype, splits=1):
                          t["sin"], t["k_pages"], t["v_pages"], H, G, d, dv, sc.rope_dims, sc.page, sc.key_chunk)
     out = torch.empty(rows, H * dv, dtype=dtype, device=q.device)
     gate_at = H * d + G * (d + dv)
-    extra = {}
+    extra = {"single_rows": True} if single_rows else {}      # the reference implementation takes no such hints
     if splits > 1:      # several workgroups share a row tile's keys and meet in a workspace
         segments = t["seg_start"].numel() - 1
-        extra = {"splits": splits, "workspace": torch.empty(o.talking_attention_workspace(rows, segments, H, dv, splits),
+        extra = {**extra, "splits": splits, "workspace": torch.empty(o.talking_attention_workspace(rows, segments, H, dv, splits),
                                                             dtype=torch.float32, device=q.device)}
     o.talking_attention(q, t["qkvg"][:, gate_at:gate_at + H], t["k_pages"], t["v_pages"], t["tables"], t["row_pos"], t["row_seg"],
                         t["seg_start"], t["talk"], t["temp"], out, H, G, d, dv, sc.page, scale, chunk, sc.key_chunk, sc.max_pos, **extra)
@@ -225,11 +225,17 @@ SHAPES = [(4, 2, 32, 16, 24, 8, 16), (6, 3, 64, 64, 40, 16, 32), (12, 4, 32, 16,
 SEGMENTS = [(0, 50), (37, 1), (23, 30), (79, 2), (80, 1), (95, 18), (0, 1), (120, 1), (47, 1), (48, 1), (2, 2), (199, 1)]
 
 
+# a decode step: one row a request, right before, on and after the edges of chunks, pages and key blocks
+SINGLE_ROWS = [(0, 1), (1, 1), (15, 1), (16, 1), (39, 1), (40, 1), (63, 1), (64, 1), (79, 1), (80, 1), (127, 1), (128, 1), (199, 1), (33, 1)]
+
+
+@pytest.mark.parametrize("rows", ["mixed", "single"])
 @pytest.mark.parametrize("fast", [True, False, 2, 5])      # a number: the matrix-core kernel with that many workgroups a row tile
 @pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
 @pytest.mark.parametrize("shape", SHAPES)
-def test_mixed_head_attention_over_pages(ops, ref, shape, dtype, fast):
+def test_mixed_head_attention_over_pages(ops, ref, shape, dtype, fast, rows):
     H, G, d, dv, chunk, page, rope_dims = shape
+    SEGMENTS = SINGLE_ROWS if rows == "single" else globals()["SEGMENTS"]
     splits, fast = (fast, True) if fast not in (True, False) else (1, fast)
     if dtype == torch.float32 and (not fast or splits > 1):
         pytest.skip("float32 has one kernel")
@@ -248,7 +254,7 @@ def test_mixed_head_attention_over_pages(ops, ref, shape, dtype, fast):
     ops.set_fast_kernels(fast)
     try:
         got_t = sc.tensors(DEV)
-        got_q, got = run_mixer_kernels(ops, got_t, sc, chunk, scale, dtype, splits)
+        got_q, got = run_mixer_kernels(ops, got_t, sc, chunk, scale, dtype, splits, single_rows=rows == "single")
         torch.cuda.synchronize()
     finally:
         ops.set_fast_kernels(True)

@@ -105,7 +105,9 @@ talking_tile_kernel(const TalkArgs p) {
     int *ptab = (int *)(stage + ((stage_elems + 7) & ~(size_t)7));
     __shared__ int starts[kMaxSegsLds + 1];
     int seg, first, nrows;
-    if (!find_tile(p, blockIdx.x, starts, seg, first, nrows)) return;
+    // the last tiles of a prompt see the most keys: they start first, so that the short ones fill the gaps at the end
+    const int tile = gridDim.x - 1 - blockIdx.x;
+    if (!find_tile(p, tile, starts, seg, first, nrows)) return;
     const int S = p.splits, split = blockIdx.y;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c = lane & 15, g = lane >> 4;
@@ -374,7 +376,7 @@ talking_tile_kernel(const TalkArgs p) {
     __syncthreads();
     if (S > 1) {
         // this workgroup's share of the tile: maxima and sums [heads][16], unnormalised outputs [16][heads][v_dim]
-        float *part = p.ws + ((size_t)blockIdx.x * S + split) * part_floats(H, DV);
+        float *part = p.ws + ((size_t)tile * S + split) * part_floats(H, DV);
         float *part_o = part + 2 * kTileRows * H;
 #pragma unroll
         for (int h = 0; h < HMAX; h++) {

@@ -650,37 +650,57 @@ talking_decode_kernel(const TalkArgs p) {
     }
 }
 
-// The shares of a decode row's workgroups into its output, a workgroup a (request, head).
-__global__ void __launch_bounds__(64) talking_decode_merge_kernel(const TalkArgs p) {
+// The shares of a decode row's workgroups into its output, a workgroup a (request, head): eight groups of 32 threads take
+// every eighth share each (a thread four value lanes), then the eight partial merges meet in LDS.
+__global__ void __launch_bounds__(kThreads) talking_decode_merge_kernel(const TalkArgs p) {
+    __shared__ float gm[8], gl[8];
+    __shared__ __attribute__((aligned(16))) float go[8][128];
     const int seg = blockIdx.x, h = blockIdx.y, H = p.heads, DV = p.v_dim, S = p.splits;
     const int r = p.seg_start[seg];
     if (p.row_seg[r] < 0) return;      // a padding row: the decode kernel has written zeros
     const size_t per = decode_part_floats(H, DV);
     const float *parts = p.ws + (size_t)seg * S * per;
-    for (int d4 = 4 * threadIdx.x; d4 < DV; d4 += 4 * 64) {
-        float m = -INFINITY;
-#pragma unroll 4
-        for (int s = 0; s < S; s++) m = fmaxf(m, parts[s * per + h]);
-        float l = 0.f;
-        f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
-        if (m > -INFINITY) {
-#pragma unroll 4
-            for (int s = 0; s < S; s++) {
-                const float *part = parts + s * per;
-                const float w = __expf(part[h] - m);
-                l += part[H + h] * w;
-                const f32x4_t o4 = *(const f32x4_t *)(part + 2 * H + (size_t)h * DV + d4);
+    const int sg = threadIdx.x >> 5, d4 = 4 * (threadIdx.x & 31);
+    float m = -INFINITY, l = 0.f;
+    f32x4_t acc = {0.f, 0.f, 0.f, 0.f};
+    for (int s = sg; s < S; s += 8) {
+        const float *part = parts + s * per;
+        const float ms = part[h], ls = part[H + h];
+        f32x4_t o4 = {0.f, 0.f, 0.f, 0.f};
+        if (d4 < DV) o4 = *(const f32x4_t *)(part + 2 * H + (size_t)h * DV + d4);
+        if (ms == -INFINITY) continue;      // a share that saw no key
+        const float m_new = fmaxf(m, ms);
+        const float a = __expf(m - m_new), w = __expf(ms - m_new);      // m = -inf: a = 0
+        l = l * a + ls * w;
 #pragma unroll
-                for (int e = 0; e < 4; e++) acc[e] = fmaf(o4[e], w, acc[e]);
-            }
-        }
-        float f = l > 0.f ? 1.0f / l : 0.f;
-        if (p.gate != nullptr) f *= 1.0f / (1.0f + __expf(-(float)p.gate[(size_t)r * p.gate_stride + h]));
-        bf16x4_t r4;
-#pragma unroll
-        for (int e = 0; e < 4; e++) r4[e] = (bf16_t)(acc[e] * f);
-        *(bf16x4_t *)(p.out + (size_t)r * H * DV + (size_t)h * DV + d4) = r4;
+        for (int e = 0; e < 4; e++) acc[e] = acc[e] * a + o4[e] * w;
+        m = m_new;
     }
+    if ((threadIdx.x & 31) == 0) { gm[sg] = m; gl[sg] = l; }
+    if (d4 < DV) *(f32x4_t *)&go[sg][d4] = acc;
+    __syncthreads();
+    if (sg != 0 || d4 >= DV) return;
+    float mt = -INFINITY;
+#pragma unroll
+    for (int k = 0; k < 8; k++) mt = fmaxf(mt, gm[k]);
+    float lt = 0.f;
+    f32x4_t tot = {0.f, 0.f, 0.f, 0.f};
+    if (mt > -INFINITY) {
+#pragma unroll
+        for (int k = 0; k < 8; k++) {
+            const float w = __expf(gm[k] - mt);      // a group without a share: e^-inf = 0
+            lt += gl[k] * w;
+            const f32x4_t o4 = *(const f32x4_t *)&go[k][d4];
+#pragma unroll
+            for (int e = 0; e < 4; e++) tot[e] = fmaf(o4[e], w, tot[e]);
+        }
+    }
+    float f = lt > 0.f ? 1.0f / lt : 0.f;
+    if (p.gate != nullptr) f *= 1.0f / (1.0f + __expf(-(float)p.gate[(size_t)r * p.gate_stride + h]));
+    bf16x4_t r4;
+#pragma unroll
+    for (int e = 0; e < 4; e++) r4[e] = (bf16_t)(tot[e] * f);
+    *(bf16x4_t *)(p.out + (size_t)r * H * DV + (size_t)h * DV + d4) = r4;
 }
 
 // 1: not taken
@@ -696,7 +716,7 @@ int launch_decode(const TalkArgs &a, hipStream_t stream) {
     else hipLaunchKernelGGL(talking_decode_kernel<8>, dim3(a.num_segs, a.splits), dim3(kThreads), lds, stream, a);
     int rc = fllm_check_launch("talking_attention (decode rows)");
     if (rc == 0 && a.splits > 1) {
-        hipLaunchKernelGGL(talking_decode_merge_kernel, dim3(a.num_segs, H), dim3(64), 0, stream, a);
+        hipLaunchKernelGGL(talking_decode_merge_kernel, dim3(a.num_segs, H), dim3(kThreads), 0, stream, a);
         rc = fllm_check_launch("talking_attention (decode merge)");
     }
     return rc;

@@ -494,7 +494,7 @@ talking_decode_kernel(const TalkArgs p) {
     const int seg = blockIdx.x, split = blockIdx.y, S = p.splits;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int c = lane & 15, g = lane >> 4;
-    const int r = p.seg_start[seg];
+    const int r = seg;      // every segment has one row: its first row is its own number, no lookup to wait for
     const size_t out_row = (size_t)H * DV;
     if (p.row_seg[r] < 0) {   // padding rows of a captured step
         if (split == 0)
@@ -523,6 +523,13 @@ talking_decode_kernel(const TalkArgs p) {
 
     for (int b = 0; b < my_blocks; b++) {
         const int kb = kb_start + kKeyBlock * (split + S * b);
+        // the pages of the keys whose values this lane takes in step 3: asked for now, so that step 3 waits for no lookup
+        int vpage[2];
+#pragma unroll
+        for (int s2 = 0; s2 < 2; s2++) {
+            const int key8 = kb + 32 * s2 + 8 * g;
+            vpage[s2] = key8 <= pos ? tbl[key8 / PS] : 0;
+        }
         // ---- 1. raw scores of this wave's 16 keys, a key/value head at a time
         if (kb + 16 * wave <= pos) {
             const int key = kb + 16 * wave + c;
@@ -602,7 +609,7 @@ talking_decode_kernel(const TalkArgs p) {
                                 const int key8 = kb + 32 * s2 + 8 * g;
                                 bf16x8_t vf = vzero;
                                 if (key8 <= pos) {
-                                    const bf16x8_t v8 = *(const bf16x8_t *)(p.v_pages + (((size_t)tbl[key8 / PS] * G + kvh) * DV + 16 * t + c) * PS + key8 % PS);
+                                    const bf16x8_t v8 = *(const bf16x8_t *)(p.v_pages + (((size_t)vpage[s2] * G + kvh) * DV + 16 * t + c) * PS + key8 % PS);
 #pragma unroll
                                     for (int e = 0; e < 8; e++) vf[e] = key8 + e <= pos ? v8[e] : (bf16_t)0.f;   // slots past the last token hold anything
                                 }
@@ -656,7 +663,7 @@ __global__ void __launch_bounds__(kThreads) talking_decode_merge_kernel(const Ta
     __shared__ float gm[8], gl[8];
     __shared__ __attribute__((aligned(16))) float go[8][128];
     const int seg = blockIdx.x, h = blockIdx.y, H = p.heads, DV = p.v_dim, S = p.splits;
-    const int r = p.seg_start[seg];
+    const int r = seg;
     if (p.row_seg[r] < 0) return;      // a padding row: the decode kernel has written zeros
     const size_t per = decode_part_floats(H, DV);
     const float *parts = p.ws + (size_t)seg * S * per;

@@ -58,6 +58,27 @@ def test_the_line_of_a_short_run():
 
 
 @pytest.mark.gpu
+def test_the_line_of_another_design_beside_its_closest_model():
+    """`--design menitar`: both models at equal sizes, decode at three batches and a prompt each, the kernels of a step."""
+    done = run_bench("--design", "menitar", "--design-size", "small", "--layers", "3", "--steps", "6", "--warmup", "2",
+                     "--repeats", "1")
+    assert done.returncode == 0, done.stderr[-2000:]
+    lines = done.stdout.strip().splitlines()
+    assert len(lines) == 1
+    line = json.loads(lines[0])
+    assert line["layer_runs"] == 4 and line["sizes"]["layers"] == 3 and line["dtype"] == "bf16"
+    for model in ("menitar", "llama"):
+        got = line[model]
+        assert set(got) >= {"decode_b1", "decode_b8", "decode_b64", "prefill", "kernels"}
+        assert got["decode_b64"]["tokens_per_s"] > got["decode_b1"]["tokens_per_s"] > 0
+        assert abs(got["prefill"]["tokens_per_s"] - 2048 / (got["prefill"]["ms"] * 1e-3)) < 0.01 * got["prefill"]["tokens_per_s"]
+        assert set(got["kernels"]) == {"prefill_us", "decode_b8_us"}
+    # the decode step of the new design runs its own matrix-core attention and the fused forms of its products
+    names = " ".join(line["menitar"]["kernels"]["decode_b8_us"])
+    assert "talking_decode_kernel" in names and "glu_clamped" not in names and "rmsnorm_pair" not in names
+
+
+@pytest.mark.gpu
 def test_the_smoke_run_of_the_entry_file():
     """`__graft_entry__.smoke()` in a process of its own, as it is run: a few tokens of a tiny random model on the
     device against the plain implementation."""

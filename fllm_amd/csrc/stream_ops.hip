@@ -49,6 +49,26 @@ glu_clamped_kernel(const T *__restrict__ gu, T *__restrict__ out, int inter, flo
     o[c] = from_f32<T>(gf / (1.0f + expf(-alpha * gf)) * (uf + up_offset));
 }
 
+// the same for bfloat16 rows whose width is a multiple of 8: a thread takes 8 neighbours, 16 bytes of gate and of up
+__global__ void __launch_bounds__(kBlock)
+glu_clamped_vec_kernel(const bf16_t *__restrict__ gu, bf16_t *__restrict__ out, int inter, float limit, float alpha, float up_offset) {
+    const size_t r = blockIdx.y;
+    const int c = (blockIdx.x * kBlock + threadIdx.x) * 8;
+    if (c >= inter) return;
+    const bf16x8_t g8 = *(const bf16x8_t *)(gu + r * 2 * inter + c), u8 = *(const bf16x8_t *)(gu + r * 2 * inter + inter + c);
+    bf16x8_t o8;
+#pragma unroll
+    for (int e = 0; e < 8; e++) {
+        float gf = (float)g8[e], uf = (float)u8[e];
+        if (limit > 0.f) {
+            gf = fminf(gf, limit);
+            uf = fminf(fmaxf(uf, -limit), limit);
+        }
+        o8[e] = (bf16_t)(gf / (1.0f + expf(-alpha * gf)) * (uf + up_offset));
+    }
+    *(bf16x8_t *)(out + r * inter + c) = o8;
+}
+
 __global__ void __launch_bounds__(kBlock) scale_kernel(float *__restrict__ x, size_t total, float scale) {
     for (size_t i = (size_t)blockIdx.x * kBlock + threadIdx.x; i < total; i += (size_t)gridDim.x * kBlock) x[i] *= scale;
 }
@@ -100,6 +120,9 @@ extern "C" int fllm_glu_clamped(const void *gate_up, void *out, int rows, int in
     if (dtype == FLLM_F32)
         hipLaunchKernelGGL(glu_clamped_kernel<float>, grid, dim3(kBlock), 0, stream, (const float *)gate_up, (float *)out, inter,
                            limit, alpha, up_offset);
+    else if (dtype == FLLM_BF16 && inter % 8 == 0 && (((uintptr_t)gate_up | (uintptr_t)out) & 15) == 0)
+        hipLaunchKernelGGL(glu_clamped_vec_kernel, dim3((inter / 8 + kBlock - 1) / kBlock, rows), dim3(kBlock), 0, stream,
+                           (const bf16_t *)gate_up, (bf16_t *)out, inter, limit, alpha, up_offset);
     else if (dtype == FLLM_BF16)
         hipLaunchKernelGGL(glu_clamped_kernel<bf16_t>, grid, dim3(kBlock), 0, stream, (const bf16_t *)gate_up, (bf16_t *)out, inter,
                            limit, alpha, up_offset);

@@ -48,6 +48,8 @@ qk_norm_rope_store_kernel(const T *__restrict__ qkv, int ld, const float *__rest
     const int pos = row_pos[r];
     const int nq = heads * k_dim, nk = kv_heads * k_dim, nv = kv_heads * v_dim;
     const T *q = qkv + r * ld, *k = q + nq, *v = k + nk;
+    // asked for before the sums, so that the lookup waits beside them and not behind them
+    const int page = store_kv ? tables[(size_t)seg * table_stride + pos / page_size] : 0, off = pos % page_size;
     float sq = 0.f, sk = 0.f;
     for (int c = threadIdx.x; c < nq; c += kBlock) { const float a = to_f32<T>(q[c]); sq += a * a; }
     for (int c = threadIdx.x; c < nk; c += kBlock) { const float a = to_f32<T>(k[c]); sk += a * a; }
@@ -56,7 +58,6 @@ qk_norm_rope_store_kernel(const T *__restrict__ qkv, int ld, const float *__rest
     const float inv_q = 1.0f / sqrtf(sq / (float)nq + eps), inv_k = 1.0f / sqrtf(sk / (float)nk + eps);
     const int half = rope_dims / 2;
     const float *cs = cos_table + (size_t)pos * half, *sn = sin_table + (size_t)pos * half;
-    const int page = store_kv ? tables[(size_t)seg * table_stride + pos / page_size] : 0, off = pos % page_size;
     for (int idx = threadIdx.x; idx < nq + (store_kv ? nk : 0); idx += kBlock) {
         const bool is_q = idx < nq;
         const int e = is_q ? idx : idx - nq;

@@ -42,8 +42,15 @@ S = config(128, 160, [layer(8, 2, 64, 32, chunk=80, rot=(32, 25000.0), ff=192),
                       layer(8, 2, 64, 32, chunk=80, rot=(32, 25000.0), ff=192)], loop=(1, 3, 2))
 # T: twelve heads (the wider instance of the matrix-core kernel), a chunk of one page
 T = config(64, 72, [layer(12, 4, 32, 16, chunk=16, rot=(32, 3000.0), ff=96)])
-CONFIGS = {"P": P, "Q": Q, "R": R, "S": S, "T": T}
-PAGE_SIZES = {"P": 8, "Q": 16, "R": 8, "S": 16, "T": 16}
+# U: sizes that are multiples of nothing (width, vocabulary, feed-forward), heads of 24 lanes with values of 20, three heads
+# on one key/value head, a chunk of 7 positions, a loop over every layer
+U = config(68, 77, [layer(3, 1, 24, 20, chunk=7, rot=(10, 77.0), ff=50, limit=0.9),
+                    layer(3, 1, 24, 20, chunk=7, rot=(10, 77.0), ff=50, limit=0.9)], loop=(0, 2, 2), embedding_scale=2.0, logit_scale=3.0)
+# V: twenty heads on four key/value heads (more heads than the row-tile kernel holds: prompts run the plain kernel, decode
+# steps the matrix-core one), values wider than keys
+V = config(80, 90, [layer(20, 4, 32, 48, chunk=48, rot=(32, 1000.0), ff=120)])
+CONFIGS = {"P": P, "Q": Q, "R": R, "S": S, "T": T, "U": U, "V": V}
+PAGE_SIZES = {"P": 8, "Q": 16, "R": 8, "S": 16, "T": 16, "U": 16, "V": 16}
 
 
 def bf16_round(a):

@@ -80,7 +80,7 @@ def test_the_loader_names_what_does_not_fit():
     assert [w[0] for w in err.value.wrong_shape] == ["l0.mix.talk"]
 
 
-@pytest.mark.parametrize("name,lengths", [("P", [5, 30, 61]), ("Q", [45, 83]), ("R", [9, 50]), ("S", [100, 37])])
+@pytest.mark.parametrize("name,lengths", [("P", [5, 30, 61]), ("Q", [45, 83]), ("R", [9, 50]), ("S", [100, 37]), ("U", [20, 51])])
 @pytest.mark.parametrize("family", ["whole", "last", "portions", "mixed"])
 def test_every_way_of_cutting_gives_the_plain_logits(tmp_path, name, lengths, family):
     vocab = mc.CONFIGS[name]["vocab"]

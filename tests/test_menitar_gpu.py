@@ -219,7 +219,8 @@ def run_mixer_kernels(o, t, sc, chunk, scale, dtype, splits=1, single_rows=False
 # heads, kv heads, key size, value size, chunk, page, rotated lanes
 SHAPES = [(4, 2, 32, 16, 24, 8, 16), (6, 3, 64, 64, 40, 16, 32), (12, 4, 32, 16, 16, 16, 32), (2, 1, 20, 12, None, 8, 0),
           (8, 2, 64, 32, 80, 16, 32), (16, 16, 32, 32, 33, 32, 8), (3, 3, 32, 32, 40, 16, 32), (5, 1, 128, 128, 100, 64, 64),
-          (8, 8, 256, 64, None, 16, 64)]
+          (8, 8, 256, 64, None, 16, 64), (4, 2, 48, 24, 50, 16, 16), (4, 2, 64, 40, 30, 16, 64), (20, 4, 32, 48, 64, 16, 16),
+          (32, 8, 64, 64, 70, 8, 32)]
 # (held, new) per request: prompts from the first token, portions that begin inside a chunk and cross its edge, single
 # rows right before, on and after an edge, two-token portions
 SEGMENTS = [(0, 50), (37, 1), (23, 30), (79, 2), (80, 1), (95, 18), (0, 1), (120, 1), (47, 1), (48, 1), (2, 2), (199, 1)]
@@ -342,7 +343,7 @@ def test_the_matrix_core_kernel_is_the_one_that_runs(ops):
 # the engine
 # ---------------------------------------------------------------------------------------------
 LENGTHS = {"P": [5, 30, 61, 100, 49], "Q": [45, 83, 161, 2, 120], "R": [9, 50, 300, 130], "S": [100, 37, 250, 81, 160],
-           "T": [3, 17, 64, 33, 150]}
+           "T": [3, 17, 64, 33, 150], "U": [31, 2, 75, 120], "V": [40, 97, 130, 7]}
 # about three times the largest error any case here has shown on the MI355X (float32 8.4e-7, bfloat16 8.6e-3)
 TOL = {"float32": 3e-6, "bfloat16": 2.5e-2}
 
@@ -377,7 +378,7 @@ def check(got, plain, dtype, what):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["P", "Q", "R", "S", "T"])
+@pytest.mark.parametrize("name", ["P", "Q", "R", "S", "T", "U", "V"])
 @pytest.mark.parametrize("family", ["whole", "last40", "portions", "mixed"])
 def test_replay(models, tmp_path, name, dtype, family):
     folder, cfg, requests, plain, _ = models[name]

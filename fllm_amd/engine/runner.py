@@ -68,7 +68,7 @@ class ModelRunner:
                  ops=None, typed_config=None, use_graphs: bool = True, max_step_tokens: Optional[int] = None,
                  decode_weight_tiles="auto", consume_tensors: bool = False):
         """`num_pages`: pages of every cache group (one number) or of each group (a list); by default what
-        `max_tokens` tokens need, else what fits on the card.  `max_step_tokens`: the most tokens of one request
+        `max_tokens` tokens need, else what fits on the device.  `max_step_tokens`: the most tokens of one request
         that a step may bring (more are refused); with it, groups that keep a window of keys are made no larger than
         `max_requests` requests can fill.  `decode_weight_tiles`: True, False or "auto" (while memory is plentiful): the
         matrices whose products add into the residual stream keep a second, tile-major copy for decode steps
@@ -144,7 +144,7 @@ class ModelRunner:
         return caps
 
     def _pages_that_fit(self, utilization: float, max_requests: int) -> List[int]:
-        """Pages for what is left of the card after the weights: window groups get what `max_requests` requests
+        """Pages for what is left of the device memory after the weights: window groups get what `max_requests` requests
         can fill, the other groups share the rest equally (a token needs a page of each), capped likewise."""
         per_page = self.model.cache_bytes_per_page(self.page_size)
         caps = self._page_caps(max_requests)

@@ -1,6 +1,11 @@
 """Menitar on the MI355X: each of its kernels alone against tests/reference_ops.py (float64), then the engine's steps
 however a request is cut and batched, captured decode steps and greedy generation against tests/plain_menitar.py."""
 
+import json
+import os
+import subprocess
+import sys
+
 import numpy as np
 import pytest
 import torch
@@ -501,3 +506,23 @@ def test_greedy_generation_through_the_scheduler(models, name):
         top = np.sort(logits)[-2:]
         if top[1] - top[0] > 0.1 * np.abs(logits).max():
             assert o[0] == int(np.argmax(logits))
+
+
+def test_the_command_line_generates_and_samples(models):
+    """`python -m fllm_amd run` on a Menitar folder: greedy tokens are the plain implementation's, and the sampling
+    options (temperature, top-k, top-p, penalties, several answers, log-probabilities, the prefix cache) run."""
+    folder, cfg, _, _, w64 = models["S"]
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    prompt = mc.random_ids(30, cfg["vocab"], 4)
+    cmd = [sys.executable, "-m", "fllm_amd", "run", folder, "--prompt-ids", ",".join(map(str, prompt)), "--max-tokens", "8",
+           "--dtype", "float32", "--ctx", "256", "--kv-blocks", "16", "--max-seqs", "2"]
+    proc = subprocess.run(cmd, cwd=root, capture_output=True, text=True, timeout=110)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    record = json.loads(proc.stdout.strip().splitlines()[0])
+    assert record["finish_reason"] == "length" and record["token_ids"] == plain_menitar.greedy(cfg, w64, prompt, 8)
+    flags = ["--temperature", "0.8", "--top-k", "20", "--top-p", "0.9", "--seed", "3", "--repeat-penalty", "1.3", "--n", "2",
+             "--logprobs", "2", "--prefix-cache", "--dtype", "bfloat16"]
+    proc = subprocess.run(cmd + flags, cwd=root, capture_output=True, text=True, timeout=110)
+    assert proc.returncode == 0, proc.stderr[-2000:]
+    records = [json.loads(line) for line in proc.stdout.strip().splitlines()]
+    assert len(records) == 2 and all(len(r["token_ids"]) == 8 for r in records)

@@ -2,6 +2,7 @@ from .spec import ConfigError, LayerSpec, ModelSpec, PartSpec, RunEntry, default
 from .files import read_config_json
 from .llama import LlamaConfig, RopeScaling
 from .menitar import MenitarConfig
+from .purivik import PurivikConfig
 
 __all__ = ["ConfigError", "LayerSpec", "ModelSpec", "PartSpec", "RunEntry", "default_run_order",
-           "LlamaConfig", "MenitarConfig", "RopeScaling", "read_config_json"]
+           "LlamaConfig", "MenitarConfig", "PurivikConfig", "RopeScaling", "read_config_json"]

@@ -133,18 +133,21 @@ int fllm_add_residual(float *residual, const void *branch, int rows, int width, 
 int fllm_swiglu(const void *gate_up, void *out, int rows, int inter, int dtype, hipStream_t stream);
 
 // Rotates the query and key heads of qkv rows in place and stores keys and values in pages.
-// qkv: [rows, (heads + 2 kv_heads) * head_dim]; row r belongs to segment row_seg[r] at position
-// row_pos[r]; its page is tables[row_seg[r] * table_stride + row_pos[r] / page_size].
-// K pages: [page][kv_head][token][head_dim]; V pages: [page][kv_head][head_dim][token].
+// qkv: [rows, (heads + kv_heads) * head_dim + kv_heads * v_dim] (values may have a width of their own); row r belongs to
+// segment row_seg[r] at position row_pos[r]; its page is tables[row_seg[r] * table_stride + row_pos[r] / page_size].
+// K pages: [page][kv_head][head_dim / 8][token][8]; V pages: [page][kv_head][v_dim][token].
 // pairing 0: lanes (l, l + rope_dims/2); 1: lanes (2l, 2l + 1).  store_kv 0 leaves the pages alone.
 int fllm_rope_kv_store(void *qkv, const int32_t *row_pos, const int32_t *row_seg, const int32_t *tables,
                        int table_stride, const float *cos_table, const float *sin_table, int table_positions,
                        void *k_pages, void *v_pages, int num_pages, int rows, int heads, int kv_heads, int head_dim,
-                       int rope_dims, int pairing, int page_size, int dtype, int store_kv, hipStream_t stream);
+                       int v_dim, int rope_dims, int pairing, int page_size, int key_chunk, int dtype, int store_kv,
+                       hipStream_t stream);
 
 // Causal attention of each row over the pages of its segment: keys at positions
-// [max(0, pos - window + 1), pos] (window <= 0: from 0).  q: rows of `q_stride` elements, head h at
-// h * head_dim.  out: [rows, heads * head_dim].  Rows of a segment are consecutive in the batch, at
+// [max(0, pos - window + 1), pos] (window <= 0: from 0), and with chunk > 0 none before pos - pos % chunk (the start of
+// the row's own chunk of positions).  q: rows of `q_stride` elements, head h at h * head_dim.  Values have `v_dim` lanes
+// a head; out: [rows, heads * v_dim].  Keys lie in chunks of `key_chunk` values inside a page (8, or 1 for head sizes
+// that are no multiple of 8).  The matrix-core kernels take v_dim == head_dim and chunks of 8; the rest runs the plain kernel.  Rows of a segment are consecutive in the batch, at
 // consecutive positions; seg_start[s] is the first row of segment s (seg_start[num_segs] = rows).
 // `max_context` bounds pos + 1.  The segments from `single_from` on have one row each (0: every segment, a decode
 // step; num_segs: none is known to): rows of long contexts among them are split over workgroups, which portions
@@ -152,8 +155,8 @@ int fllm_rope_kv_store(void *qkv, const int32_t *row_pos, const int32_t *row_seg
 // the number of single rows).
 int fllm_attention(const void *q, int q_stride, const void *k_pages, const void *v_pages, const int32_t *tables,
                    int table_stride, const int32_t *row_pos, const int32_t *row_seg, const int32_t *seg_start,
-                   int num_segs, void *out, int rows, int heads, int kv_heads, int head_dim, int page_size,
-                   int num_pages, float scale, int window, int dtype, int max_context, int single_from,
+                   int num_segs, void *out, int rows, int heads, int kv_heads, int head_dim, int v_dim, int page_size,
+                   int num_pages, float scale, int window, int chunk, int key_chunk, int dtype, int max_context, int single_from,
                    void *workspace, size_t workspace_bytes, hipStream_t stream);
 size_t fllm_attention_workspace_bytes(int rows, int heads, int kv_heads, int head_dim, int max_context);
 // The same attention with a bias on every score that depends on the distance alone: score(row, key) = q . k * scale +
@@ -294,6 +297,24 @@ int fllm_talking_attention(const void *q, const void *gate, int gate_stride, con
 // `ws`, float32, at least fllm_talking_attention_workspace(...) floats; the plain kernels ignore both.  `single_rows`: the
 // caller knows that every segment has one row (a decode step), which has a matrix-core kernel of its own.
 size_t fllm_talking_attention_workspace(int rows, int num_segs, int heads, int v_dim, int splits);
+
+// A branch that is normed on its way into the float32 residual stream: v = the sum of the row's `parts` partial branches
+// (branch: [rows, parts, width] of `branch_dtype`), x[r] += v * rsqrt(mean(v^2) + eps) * gain (normalize 0: x[r] += v * gain).
+// With next_w, next_out[r] = rmsnorm(x[r]) * next_w with next_eps (of `next_dtype`) as well.
+int fllm_postnorm_add(float *x, const void *branch, int branch_dtype, int parts, const float *gain, float eps, int normalize,
+                      const float *next_w, float next_eps, void *next_out, int next_dtype, int rows, int width, hipStream_t stream);
+
+// Routed experts, plain kernels.  fllm_route_topk: score = sigmoid(w_router h) in float32 ([E, K] beside rows [rows, K] of
+// `dtype`, row stride ldh); ids[r, k] / weights[r, k] = the expert with the k-th largest score of row r (the lower index
+// among equals) and that score.  fllm_experts_gate_up: for every (row, pick) pair, act[pair] = a(g) * (u + up_offset) with
+// g, u = the gate and up rows of the picked expert times (h[row] * weight), clamped as in fllm_glu_clamped;
+// w_gate_up = [E][2 inter][K].  fllm_experts_down: out[pair] = w_down[e] act[pair], float32; w_down = [E][N][inter].
+int fllm_route_topk(const void *h, int ldh, const void *w_router, int rows, int K, int E, int top, int32_t *ids, float *weights,
+                    int dtype, hipStream_t stream);
+int fllm_experts_gate_up(const void *h, int ldh, const int32_t *ids, const float *weights, int rows, int top, const void *w_gate_up,
+                         int E, int inter, int K, void *act, float limit, float alpha, float up_offset, int dtype, hipStream_t stream);
+int fllm_experts_down(const void *act, const int32_t *ids, int pairs, const void *w_down, int E, int N, int inter, float *out, int dtype,
+                      hipStream_t stream);
 
 #ifdef __cplusplus
 }

@@ -48,6 +48,7 @@ struct AttnArgs {
     int ps_shift;   // page_size = 1 << ps_shift
     float scale_log2;
     int window;
+    int chunk;      // > 0: a row sees the keys of its own chunk of this many positions only (chunks counted from position 0)
     float *ws_ml;   // [rows, heads, splits, 2]
     float *ws_o;    // [rows, heads, splits, D]
     int splits, keys_per_split;
@@ -67,6 +68,15 @@ __device__ __forceinline__ bf16x8_t zero8() {
 }
 
 __device__ __forceinline__ float fast_exp2(float x) { return __builtin_amdgcn_exp2f(x); }
+
+// The first key that the row at position `pos` sees: `window` keys back (itself included) and not before the start of
+// its chunk of positions; 0 where neither bounds it.  It never falls as `pos` grows, so the first row of a tile has the
+// smallest and the last row the largest.
+__device__ __forceinline__ int first_key(int pos, int window, int chunk) {
+    int lo = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+    if (chunk > 0 && pos >= 0) lo = max(lo, pos - pos % chunk);
+    return lo;
+}
 
 // floats that one part of a shared row tile leaves for the merge (tile32 kernel): head_dim / 2 outputs, a maximum
 // and a sum for each of its lanes
@@ -154,7 +164,7 @@ attn_tile_kernel(AttnArgs p) {
     const bool rvalid = tq < ntok;
     const int prow = rvalid ? pos0 + tq : -1;
     const int head = kvh * G + hg;
-    const int lo_r = (p.window > 0 && prow - p.window + 1 > 0) ? prow - p.window + 1 : 0;
+    const int lo_r = first_key(prow, p.window, p.chunk);
     const int ps = p.page_size, psh = p.ps_shift, pmask = ps - 1, nkv = p.kv_heads;
 
     bf16x8_t qf[KD];
@@ -164,7 +174,7 @@ attn_tile_kernel(AttnArgs p) {
                         : zero8();
 
     const int p_last = pos0 + ntok - 1;
-    const int lo_tile = (p.window > 0 && pos0 - p.window + 1 > 0) ? pos0 - p.window + 1 : 0;
+    const int lo_tile = first_key(pos0, p.window, p.chunk);
     const int kbegin = (lo_tile / KT) * KT;
     const int32_t *tbl = p.tables + (size_t)seg * p.table_stride;
     const int cps = psh - 3;   // log2 of the 16-byte chunks per value row of a page
@@ -321,7 +331,7 @@ attn_tile32_kernel(AttnArgs p) {
     const bool rvalid = tq < ntok;
     const int prow = rvalid ? pos0 + tq : -1;
     const int head = kvh * G + hg;
-    const int lo_r = (p.window > 0 && prow - p.window + 1 > 0) ? prow - p.window + 1 : 0;
+    const int lo_r = first_key(prow, p.window, p.chunk);
     const int ps = p.page_size, psh = p.ps_shift, pmask = ps - 1, nkv = p.kv_heads;
     const int cps = psh - 3;        // log2 of the 16-byte chunks per value row of a page
 
@@ -332,9 +342,9 @@ attn_tile32_kernel(AttnArgs p) {
                         : zero8();
 
     const int p_last = pos0 + ntok - 1;
-    const int lo_tile = (p.window > 0 && pos0 - p.window + 1 > 0) ? pos0 - p.window + 1 : 0;
+    const int lo_tile = first_key(pos0, p.window, p.chunk);
     // from this key on every row of the workgroup sees every key up to pos0 (no window edge inside)
-    const int lo_all = (p.window > 0 && p_last - p.window + 1 > 0) ? p_last - p.window + 1 : 0;
+    const int lo_all = first_key(p_last, p.window, p.chunk);
     int kbegin = (lo_tile / KT) * KT;
     // Long contexts of few rows: the key tiles of this row tile are dealt out to `parts` workgroups in equal
     // stretches; a workgroup beyond that number has nothing to do.
@@ -618,7 +628,7 @@ attn_decode_kernel(AttnArgs p, int qtiles) {
     const bool qvalid = hg < G && seg >= 0;
     const int head = kvh * G + (hg < G ? hg : 0);
     const int n = seg >= 0 ? p.row_pos[row] + 1 : 0;
-    const int lo = (p.window > 0 && n - p.window > 0) ? n - p.window : 0;
+    const int lo = first_key(n - 1, p.window, p.chunk);
     const int ps = p.page_size, psh = p.ps_shift, pmask = ps - 1, nkv = p.kv_heads;
     const int first = (lo / 32) * 32;
     const int begin = first + split * p.keys_per_split;
@@ -959,10 +969,11 @@ size_t fllm_attention_bf16_workspace_bytes(int rows, int heads, int kv_heads, in
 // 0: launched, negative: error, 1: shape declined (the caller uses the plain kernel)
 int fllm_attention_bf16_fast(const void *q, int q_stride, const void *k_pages, const void *v_pages, const int32_t *tables,
                              int table_stride, const int32_t *row_pos, const int32_t *row_seg, const int32_t *seg_start,
-                             int num_segs, void *out, int rows, int heads, int kv_heads, int head_dim, int page_size,
-                             int num_pages, float scale, int window, int max_context, int single_from, void *workspace,
+                             int num_segs, void *out, int rows, int heads, int kv_heads, int head_dim, int v_dim, int page_size,
+                             int num_pages, float scale, int window, int chunk, int max_context, int single_from, void *workspace,
                              size_t workspace_bytes, hipStream_t stream) {
     if (!fllm_fast_kernels_enabled()) return 1;
+    if (v_dim != head_dim) return 1;     // these kernels read keys and values of one width
     (void)num_pages;
     if (!fast_shape(heads, kv_heads, head_dim, page_size)) return 1;
     if (q_stride % 8 != 0 || ((uintptr_t)q & 15) != 0) return 1;
@@ -988,6 +999,7 @@ int fllm_attention_bf16_fast(const void *q, int q_stride, const void *k_pages, c
     a.ps_shift = page_size == 8 ? 3 : page_size == 16 ? 4 : page_size == 32 ? 5 : 6;
     a.scale_log2 = scale * kLog2e;
     a.window = window;
+    a.chunk = chunk;
     a.ws_ml = nullptr;
     a.ws_o = nullptr;
     a.splits = 1;

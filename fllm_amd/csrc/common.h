@@ -91,6 +91,13 @@ __host__ __device__ __forceinline__ size_t key_offset(size_t page, int kv_heads,
     return ((((size_t)page * kv_heads + kvh) * (head_dim >> 3) + (d >> 3)) * page_size + token) * 8 + (d & 7);
 }
 
+// The same for keys stored in chunks of `kc` values ([kv_head][head_dim / kc][token][kc]; kc divides head_dim): 8 is the
+// order above, 1 stores a head's lanes one after the other over the tokens, for head sizes that are no multiple of 8.
+__host__ __device__ __forceinline__ size_t key_offset_chunked(size_t page, int kv_heads, int kvh, int page_size, int head_dim, int token,
+                                                              int d, int kc) {
+    return ((((size_t)page * kv_heads + kvh) * (head_dim / kc) + (d / kc)) * page_size + token) * kc + (d % kc);
+}
+
 template <typename T> __device__ __forceinline__ float to_f32(T v);
 template <> __device__ __forceinline__ float to_f32<float>(float v) { return v; }
 template <> __device__ __forceinline__ float to_f32<bf16_t>(bf16_t v) { return (float)v; }

@@ -146,7 +146,7 @@ __global__ void __launch_bounds__(kBlock)
 rope_kv_store_kernel(T *__restrict__ qkv, const int32_t *__restrict__ row_pos, const int32_t *__restrict__ row_seg,
                      const int32_t *__restrict__ tables, int table_stride, const float *__restrict__ cos_table,
                      const float *__restrict__ sin_table, T *__restrict__ k_pages, T *__restrict__ v_pages, int heads,
-                     int kv_heads, int head_dim, int rope_dims, int pairing, int page_size, int store_kv) {
+                     int kv_heads, int head_dim, int v_dim, int rope_dims, int pairing, int page_size, int key_chunk, int store_kv) {
     const int r = blockIdx.x;
     const int seg = row_seg[r];
     if (seg < 0) return;   // padding row
@@ -154,7 +154,7 @@ rope_kv_store_kernel(T *__restrict__ qkv, const int32_t *__restrict__ row_pos, c
     const int half = rope_dims / 2;
     const float *cs = cos_table + (size_t)pos * half;
     const float *sn = sin_table + (size_t)pos * half;
-    T *row = qkv + (size_t)r * (heads + 2 * kv_heads) * head_dim;
+    T *row = qkv + (size_t)r * ((size_t)(heads + kv_heads) * head_dim + (size_t)kv_heads * v_dim);
 
     // queries, in place
     for (int i = threadIdx.x; i < heads * half; i += kBlock) {
@@ -179,18 +179,18 @@ rope_kv_store_kernel(T *__restrict__ qkv, const int32_t *__restrict__ row_pos, c
         const int ia = pairing ? 2 * l : l, ib = pairing ? 2 * l + 1 : l + half;
         const T *head = krow + (size_t)h * head_dim;
         const float a = to_f32<T>(head[ia]), b = to_f32<T>(head[ib]);
-        k_pages[key_offset(page, kv_heads, h, page_size, head_dim, off, ia)] = from_f32<T>(a * cs[l] - b * sn[l]);
-        k_pages[key_offset(page, kv_heads, h, page_size, head_dim, off, ib)] = from_f32<T>(b * cs[l] + a * sn[l]);
+        k_pages[key_offset_chunked(page, kv_heads, h, page_size, head_dim, off, ia, key_chunk)] = from_f32<T>(a * cs[l] - b * sn[l]);
+        k_pages[key_offset_chunked(page, kv_heads, h, page_size, head_dim, off, ib, key_chunk)] = from_f32<T>(b * cs[l] + a * sn[l]);
     }
     const int rest = head_dim - rope_dims;
     for (int i = threadIdx.x; i < kv_heads * rest; i += kBlock) {
         const int h = i / rest, c = rope_dims + (i - h * rest);
-        k_pages[key_offset(page, kv_heads, h, page_size, head_dim, off, c)] = krow[(size_t)h * head_dim + c];
+        k_pages[key_offset_chunked(page, kv_heads, h, page_size, head_dim, off, c, key_chunk)] = krow[(size_t)h * head_dim + c];
     }
-    // values, stored transposed inside the page: [head_dim][token]
-    for (int i = threadIdx.x; i < kv_heads * head_dim; i += kBlock) {
-        const int h = i / head_dim, c = i - h * head_dim;
-        v_pages[(((size_t)page * kv_heads + h) * head_dim + c) * page_size + off] = vrow[i];
+    // values (of v_dim lanes a head), stored transposed inside the page: [v_dim][token]
+    for (int i = threadIdx.x; i < kv_heads * v_dim; i += kBlock) {
+        const int h = i / v_dim, c = i - h * v_dim;
+        v_pages[(((size_t)page * kv_heads + h) * v_dim + c) * page_size + off] = vrow[i];
     }
 }
 
@@ -312,13 +312,14 @@ __global__ void __launch_bounds__(kBlock)
 rope_kv_store_vec_kernel(bf16_t *__restrict__ qkv, const int32_t *__restrict__ row_pos, const int32_t *__restrict__ row_seg,
                          const int32_t *__restrict__ tables, int table_stride, const float *__restrict__ cos_table,
                          const float *__restrict__ sin_table, bf16_t *__restrict__ k_pages, bf16_t *__restrict__ v_pages,
-                         int rows, int heads, int kv_heads, int head_dim, int rope_dims, int page_size, int store_kv) {
+                         int rows, int heads, int kv_heads, int head_dim, int v_dim, int rope_dims, int page_size, int store_kv) {
     const int r0 = blockIdx.x * RB;
     const int nrows = min(RB, rows - r0);
     const int half = rope_dims / 2;
     const int per_head = head_dim / 8;
     const int rot_heads = store_kv ? heads + kv_heads : heads;
-    const size_t row_elems = (size_t)(heads + 2 * kv_heads) * head_dim;
+    const size_t row_elems = (size_t)(heads + kv_heads) * head_dim + (size_t)kv_heads * v_dim;
+    const int per_head_v = v_dim / 8;
     // position (-1: padding row), page and slot of the workgroup's rows
     __shared__ int s_pos[RB], s_page[RB], s_off[RB], s_run;
     if ((int)threadIdx.x < nrows) {
@@ -362,14 +363,14 @@ rope_kv_store_vec_kernel(bf16_t *__restrict__ qkv, const int32_t *__restrict__ r
     }
     if (!store_kv) return;
     if (!run) {
-        // values, stored transposed inside the page: [head_dim][token]
-        const int v_per_row = kv_heads * per_head;
+        // values, stored transposed inside the page: [v_dim][token]
+        const int v_per_row = kv_heads * per_head_v;
         for (int it = first; it < nrows * v_per_row; it += stride) {
             const int i = RB == 1 ? 0 : it / v_per_row, t = it - i * v_per_row;
             if (s_pos[i] < 0) continue;
-            const int h = t / per_head, c = (t - h * per_head) * 8;
-            const bf16x8_t v = *(const bf16x8_t *)(qkv + (size_t)(r0 + i) * row_elems + (size_t)(heads + kv_heads + h) * head_dim + c);
-            bf16_t *dst = v_pages + (((size_t)s_page[i] * kv_heads + h) * head_dim + c) * page_size + s_off[i];
+            const int h = t / per_head_v, c = (t - h * per_head_v) * 8;
+            const bf16x8_t v = *(const bf16x8_t *)(qkv + (size_t)(r0 + i) * row_elems + (size_t)(heads + kv_heads) * head_dim + (size_t)h * v_dim + c);
+            bf16_t *dst = v_pages + (((size_t)s_page[i] * kv_heads + h) * v_dim + c) * page_size + s_off[i];
 #pragma unroll
             for (int e = 0; e < 8; e++) dst[(size_t)e * page_size] = v[e];
         }
@@ -378,34 +379,34 @@ rope_kv_store_vec_kernel(bf16_t *__restrict__ qkv, const int32_t *__restrict__ r
     // the values of the 8 tokens, one head lane at a time: 16 contiguous bytes of the transposed page
     const int page = s_page[0], off = s_off[0];
     const bf16_t *vbase = qkv + (size_t)r0 * row_elems + (size_t)(heads + kv_heads) * head_dim;
-    for (int t = first; t < kv_heads * head_dim; t += stride) {
-        const int h = t / head_dim, c = t - h * head_dim;
+    for (int t = first; t < kv_heads * v_dim; t += stride) {
+        const int h = t / v_dim, c = t - h * v_dim;
         bf16x8_t v;
 #pragma unroll
         for (int i = 0; i < 8; i++) v[i] = vbase[(size_t)(RB == 8 ? i : 0) * row_elems + t];
-        *(bf16x8_t *)(v_pages + (((size_t)page * kv_heads + h) * head_dim + c) * page_size + off) = v;
+        *(bf16x8_t *)(v_pages + (((size_t)page * kv_heads + h) * v_dim + c) * page_size + off) = v;
     }
 }
 
 extern "C" int fllm_rope_kv_store(void *qkv, const int32_t *row_pos, const int32_t *row_seg, const int32_t *tables,
                                   int table_stride, const float *cos_table, const float *sin_table, int table_positions,
                                   void *k_pages, void *v_pages, int num_pages, int rows, int heads, int kv_heads,
-                                  int head_dim, int rope_dims, int pairing, int page_size, int dtype, int store_kv,
-                                  hipStream_t stream) {
-    FLLM_REQUIRE(rows >= 0 && heads > 0 && kv_heads > 0 && head_dim > 0 && page_size > 0 && table_stride > 0,
+                                  int head_dim, int v_dim, int rope_dims, int pairing, int page_size, int key_chunk, int dtype,
+                                  int store_kv, hipStream_t stream) {
+    FLLM_REQUIRE(rows >= 0 && heads > 0 && kv_heads > 0 && head_dim > 0 && v_dim > 0 && page_size > 0 && table_stride > 0,
                  "rope_kv_store: bad sizes");
     FLLM_REQUIRE(rope_dims >= 0 && rope_dims <= head_dim && rope_dims % 2 == 0,
                  "rope_kv_store: rope_dims %d must be even and at most head_dim %d", rope_dims, head_dim);
     FLLM_REQUIRE(pairing == 0 || pairing == 1, "rope_kv_store: unknown pairing %d", pairing);
     FLLM_REQUIRE(!store_kv || (k_pages && v_pages && num_pages > 0), "rope_kv_store: pages missing");
-    FLLM_REQUIRE(head_dim % 8 == 0, "rope_kv_store: head size %d; keys lie in chunks of 8 values in a page, head sizes come in steps of 8", head_dim);
+    FLLM_REQUIRE(key_chunk > 0 && head_dim % key_chunk == 0, "rope_kv_store: keys of %d lanes cannot lie in chunks of %d", head_dim, key_chunk);
     (void)table_positions;
     if (rows == 0) return 0;
     if (dtype == FLLM_F32)
         hipLaunchKernelGGL(rope_kv_store_kernel<float>, dim3(rows), dim3(kBlock), 0, stream, (float *)qkv, row_pos, row_seg,
                            tables, table_stride, cos_table, sin_table, (float *)k_pages, (float *)v_pages, heads, kv_heads,
-                           head_dim, rope_dims, pairing, page_size, store_kv);
-    else if (dtype == FLLM_BF16 && pairing == 1 && head_dim % 8 == 0 && rope_dims % 8 == 0 && ((uintptr_t)qkv & 15) == 0 &&
+                           head_dim, v_dim, rope_dims, pairing, page_size, key_chunk, store_kv);
+    else if (dtype == FLLM_BF16 && pairing == 1 && key_chunk == 8 && head_dim % 8 == 0 && v_dim % 8 == 0 && rope_dims % 8 == 0 && ((uintptr_t)qkv & 15) == 0 &&
              ((uintptr_t)cos_table & 15) == 0 && ((uintptr_t)sin_table & 15) == 0 && (!store_kv || ((((uintptr_t)k_pages | (uintptr_t)v_pages) & 15) == 0)))
     {
         // prompt portions: 8 rows a workgroup, so that runs of 8 tokens store their values 16 bytes at a time; few rows
@@ -413,16 +414,16 @@ extern "C" int fllm_rope_kv_store(void *qkv, const int32_t *row_pos, const int32
         if (rows >= 256)
             hipLaunchKernelGGL(rope_kv_store_vec_kernel<8>, dim3((rows + 7) / 8, 4), dim3(kBlock), 0, stream, (bf16_t *)qkv, row_pos,
                                row_seg, tables, table_stride, cos_table, sin_table, (bf16_t *)k_pages, (bf16_t *)v_pages, rows,
-                               heads, kv_heads, head_dim, rope_dims, page_size, store_kv);
+                               heads, kv_heads, head_dim, v_dim, rope_dims, page_size, store_kv);
         else
             hipLaunchKernelGGL(rope_kv_store_vec_kernel<1>, dim3(rows), dim3(kBlock), 0, stream, (bf16_t *)qkv, row_pos, row_seg,
                                tables, table_stride, cos_table, sin_table, (bf16_t *)k_pages, (bf16_t *)v_pages, rows, heads,
-                               kv_heads, head_dim, rope_dims, page_size, store_kv);
+                               kv_heads, head_dim, v_dim, rope_dims, page_size, store_kv);
     }
     else if (dtype == FLLM_BF16)
         hipLaunchKernelGGL(rope_kv_store_kernel<bf16_t>, dim3(rows), dim3(kBlock), 0, stream, (bf16_t *)qkv, row_pos,
                            row_seg, tables, table_stride, cos_table, sin_table, (bf16_t *)k_pages, (bf16_t *)v_pages, heads,
-                           kv_heads, head_dim, rope_dims, pairing, page_size, store_kv);
+                           kv_heads, head_dim, v_dim, rope_dims, pairing, page_size, key_chunk, store_kv);
     else
         FLLM_REQUIRE(false, "rope_kv_store: unknown dtype %d", dtype);
     return fllm_check_launch("rope_kv_store");

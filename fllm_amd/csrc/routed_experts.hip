@@ -1,0 +1,199 @@
+// A feed-forward of many small gated layers ("experts") of which every row uses a few: the router that scores the
+// experts and picks each row's best, and the products of the picked experts, one (row, pick) pair at a time.  These are
+// the plain kernels: float32 sums in a fixed order, both element types, any sizes.  A pair's result depends on its own
+// row alone, never on the rest of the batch.
+#include "api.h"
+#include "common.h"
+
+namespace {
+
+constexpr int kBlock = 256;
+constexpr int kWaves = kBlock / kWave;
+
+// sum over the lanes' share of x . w for one weight row; x float32 in LDS, w in global memory
+template <typename T>
+__device__ __forceinline__ float lane_dot(const float *__restrict__ xs, const T *__restrict__ w, int K, int lane) {
+    float acc = 0.f;
+    for (int c = lane; c < K; c += kWave) acc = fmaf(xs[c], to_f32<T>(w[c]), acc);
+    return acc;
+}
+// bfloat16 rows whose length is a multiple of 8 and that begin on 16 bytes: 8 neighbours a load
+__device__ __forceinline__ float lane_dot8(const float *__restrict__ xs, const bf16_t *__restrict__ w, int K, int lane) {
+    float acc = 0.f;
+    for (int c = lane * 8; c < K; c += kWave * 8) {
+        const bf16x8_t w8 = *(const bf16x8_t *)(w + c);
+#pragma unroll
+        for (int e = 0; e < 8; e++) acc = fmaf(xs[c + e], (float)w8[e], acc);
+    }
+    return acc;
+}
+template <typename T> __device__ __forceinline__ float row_dot(const float *xs, const T *w, int K, int lane, bool vec);
+template <> __device__ __forceinline__ float row_dot<float>(const float *xs, const float *w, int K, int lane, bool) {
+    return wave_sum(lane_dot<float>(xs, w, K, lane));
+}
+template <> __device__ __forceinline__ float row_dot<bf16_t>(const float *xs, const bf16_t *w, int K, int lane, bool vec) {
+    return wave_sum(vec ? lane_dot8(xs, w, K, lane) : lane_dot<bf16_t>(xs, w, K, lane));
+}
+
+// Router: z = W h in float32, score = sigmoid(z) (mode 0) ; the `top` largest scores of a row, ties to the lower index;
+// weights[r, k] = the score of pick k (mode 0) .  One workgroup a row; scores through LDS.
+template <typename T>
+__global__ void __launch_bounds__(kBlock)
+route_kernel(const T *__restrict__ h, int ldh, const T *__restrict__ w, int K, int E, int top, int32_t *__restrict__ ids,
+             float *__restrict__ weights) {
+    extern __shared__ float smem[];
+    float *xs = smem;          // K
+    float *score = smem + K;   // E
+    const size_t r = blockIdx.x;
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    for (int c = threadIdx.x; c < K; c += kBlock) xs[c] = to_f32<T>(h[r * ldh + c]);
+    __syncthreads();
+    const bool vec = sizeof(T) == 2 && K % 8 == 0 && ((uintptr_t)w & 15) == 0;
+    for (int e = wave; e < E; e += kWaves) {
+        const float z = row_dot<T>(xs, w + (size_t)e * K, K, lane, vec);
+        if (lane == 0) score[e] = 1.0f / (1.0f + expf(-z));
+    }
+    __syncthreads();
+    if (wave != 0) return;
+    // one wave picks: every round the largest score not yet taken, the lowest index among equals
+    for (int k = 0; k < top; k++) {
+        float best = -INFINITY;
+        int at = 0x7fffffff;
+        for (int e = lane; e < E; e += kWave) {
+            const float s = score[e];
+            if (s > best) best = s, at = e;      // ascending e: the first of equals stays
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) {
+            const float other = __shfl_xor(best, o, kWave);
+            const int other_at = __shfl_xor(at, o, kWave);
+            if (other > best || (other == best && other_at < at)) best = other, at = other_at;
+        }
+        if (lane == 0) {
+            ids[r * top + k] = at;
+            weights[r * top + k] = best;
+            score[at] = -INFINITY;               // scores are sigmoids: nothing real is that small
+        }
+        __builtin_amdgcn_wave_barrier();
+        __threadfence_block();
+    }
+}
+
+// One (row, pick) pair a workgroup row (blockIdx.y), kCols output columns a workgroup (blockIdx.x), two a wave.
+// MODE 0: act[pair, c] = a(g) * (u + up_offset) with g, u = W_gate[e] x, W_up[e] x (clamped to `limit` when > 0),
+//         a(g) = g * sigmoid(alpha g), x = the row times the pick's weight (rounded to the element type, as a stored
+//         operand would be); w = [E][2 I][K], gate rows then up rows.
+// MODE 1: out[pair, c] = W[e][c] . x, float32; w = [E][N][K]; x = act[pair].
+constexpr int kColsPerWave = 2;
+constexpr int kCols = kWaves * kColsPerWave;
+
+template <typename T, int MODE>
+__global__ void __launch_bounds__(kBlock)
+expert_rows_kernel(const T *__restrict__ x, int ldx, const int32_t *__restrict__ ids, const float *__restrict__ weights, int top,
+                   const T *__restrict__ w, int E, int N, int K, T *__restrict__ act, float *__restrict__ out, float limit,
+                   float alpha, float up_offset) {
+    extern __shared__ float xs[];   // K
+    const size_t pair = blockIdx.y;
+    int e = ids[pair];
+    e = e < 0 ? 0 : (e >= E ? E - 1 : e);     // never outside the stack of experts
+    const int lane = threadIdx.x & (kWave - 1), wave = threadIdx.x / kWave;
+    if (MODE == 0) {
+        const float scale = weights[pair];
+        const T *src = x + (pair / top) * ldx;
+        for (int c = threadIdx.x; c < K; c += kBlock) xs[c] = to_f32<T>(from_f32<T>(to_f32<T>(src[c]) * scale));
+    } else {
+        const T *src = x + pair * ldx;
+        for (int c = threadIdx.x; c < K; c += kBlock) xs[c] = to_f32<T>(src[c]);
+    }
+    __syncthreads();
+    const bool vec = sizeof(T) == 2 && K % 8 == 0 && ((uintptr_t)w & 15) == 0;
+#pragma unroll
+    for (int j = 0; j < kColsPerWave; j++) {
+        const int c = blockIdx.x * kCols + wave * kColsPerWave + j;
+        if (c >= N) break;
+        if (MODE == 0) {
+            const T *wg = w + ((size_t)e * 2 * N + c) * K, *wu = wg + (size_t)N * K;
+            float g = row_dot<T>(xs, wg, K, lane, vec), u = row_dot<T>(xs, wu, K, lane, vec);
+            if (limit > 0.f) {
+                g = fminf(g, limit);
+                u = fminf(fmaxf(u, -limit), limit);
+            }
+            if (lane == 0) act[pair * N + c] = from_f32<T>(g / (1.0f + expf(-alpha * g)) * (u + up_offset));
+        } else {
+            const float y = row_dot<T>(xs, w + ((size_t)e * N + c) * K, K, lane, vec);
+            if (lane == 0) out[pair * N + c] = y;
+        }
+    }
+}
+
+}  // namespace
+
+extern "C" int fllm_route_topk(const void *h, int ldh, const void *w_router, int rows, int K, int E, int top, int32_t *ids,
+                               float *weights, int dtype, hipStream_t stream) {
+    FLLM_REQUIRE(rows >= 0 && K > 0 && E > 0 && top > 0 && top <= E && ldh >= K, "route_topk: bad sizes (rows %d, width %d, %d experts, %d picked)",
+                 rows, K, E, top);
+    FLLM_REQUIRE(h && w_router && ids && weights, "route_topk: operands missing");
+    const size_t smem = (size_t)(K + E) * sizeof(float);
+    FLLM_REQUIRE(smem <= 64 * 1024, "route_topk: a width of %d with %d experts does not fit into LDS", K, E);
+    if (rows == 0) return 0;
+    if (dtype == FLLM_F32)
+        hipLaunchKernelGGL(route_kernel<float>, dim3(rows), dim3(kBlock), smem, stream, (const float *)h, ldh, (const float *)w_router, K, E,
+                           top, ids, weights);
+    else if (dtype == FLLM_BF16)
+        hipLaunchKernelGGL(route_kernel<bf16_t>, dim3(rows), dim3(kBlock), smem, stream, (const bf16_t *)h, ldh, (const bf16_t *)w_router, K,
+                           E, top, ids, weights);
+    else
+        FLLM_REQUIRE(false, "route_topk: unknown dtype %d", dtype);
+    return fllm_check_launch("route_topk");
+}
+
+extern "C" int fllm_experts_gate_up(const void *h, int ldh, const int32_t *ids, const float *weights, int rows, int top,
+                                    const void *w_gate_up, int E, int inter, int K, void *act, float limit, float alpha, float up_offset,
+                                    int dtype, hipStream_t stream) {
+    FLLM_REQUIRE(rows >= 0 && top > 0 && E > 0 && inter > 0 && K > 0 && ldh >= K, "experts_gate_up: bad sizes");
+    FLLM_REQUIRE(h && ids && weights && w_gate_up && act, "experts_gate_up: operands missing");
+    FLLM_REQUIRE((size_t)K * sizeof(float) <= 64 * 1024, "experts_gate_up: a width of %d does not fit into LDS", K);
+    const long pairs = (long)rows * top;
+    FLLM_REQUIRE(pairs <= 65535 * 64L, "experts_gate_up: too many rows");
+    if (pairs == 0) return 0;
+    const size_t smem = (size_t)K * sizeof(float);
+    // at most 65,535 pairs a launch (the grid's second dimension)
+    for (long first = 0; first < pairs; first += 65535) {
+        const int count = (int)(pairs - first < 65535 ? pairs - first : 65535);
+        const dim3 grid((inter + kCols - 1) / kCols, count);
+        FLLM_REQUIRE(first % top == 0 || top == 1 || pairs <= 65535, "experts_gate_up: a launch must begin on a row");
+        if (dtype == FLLM_F32)
+            hipLaunchKernelGGL((expert_rows_kernel<float, 0>), grid, dim3(kBlock), smem, stream, (const float *)h + (first / top) * ldh, ldh,
+                               ids + first, weights + first, top, (const float *)w_gate_up, E, inter, K, (float *)act + first * inter, nullptr,
+                               limit, alpha, up_offset);
+        else if (dtype == FLLM_BF16)
+            hipLaunchKernelGGL((expert_rows_kernel<bf16_t, 0>), grid, dim3(kBlock), smem, stream, (const bf16_t *)h + (first / top) * ldh, ldh,
+                               ids + first, weights + first, top, (const bf16_t *)w_gate_up, E, inter, K, (bf16_t *)act + first * inter,
+                               nullptr, limit, alpha, up_offset);
+        else
+            FLLM_REQUIRE(false, "experts_gate_up: unknown dtype %d", dtype);
+    }
+    return fllm_check_launch("experts_gate_up");
+}
+
+extern "C" int fllm_experts_down(const void *act, const int32_t *ids, int pairs, const void *w_down, int E, int N, int inter, float *out,
+                                 int dtype, hipStream_t stream) {
+    FLLM_REQUIRE(pairs >= 0 && E > 0 && N > 0 && inter > 0, "experts_down: bad sizes");
+    FLLM_REQUIRE(act && ids && w_down && out, "experts_down: operands missing");
+    FLLM_REQUIRE((size_t)inter * sizeof(float) <= 64 * 1024, "experts_down: experts of %d lanes do not fit into LDS", inter);
+    if (pairs == 0) return 0;
+    const size_t smem = (size_t)inter * sizeof(float);
+    for (long first = 0; first < pairs; first += 65535) {
+        const int count = (int)(pairs - first < 65535 ? pairs - first : 65535);
+        const dim3 grid((N + kCols - 1) / kCols, count);
+        if (dtype == FLLM_F32)
+            hipLaunchKernelGGL((expert_rows_kernel<float, 1>), grid, dim3(kBlock), smem, stream, (const float *)act + first * inter, inter,
+                               ids + first, nullptr, 1, (const float *)w_down, E, N, inter, nullptr, out + first * N, 0.f, 0.f, 0.f);
+        else if (dtype == FLLM_BF16)
+            hipLaunchKernelGGL((expert_rows_kernel<bf16_t, 1>), grid, dim3(kBlock), smem, stream, (const bf16_t *)act + first * inter, inter,
+                               ids + first, nullptr, 1, (const bf16_t *)w_down, E, N, inter, nullptr, out + first * N, 0.f, 0.f, 0.f);
+        else
+            FLLM_REQUIRE(false, "experts_down: unknown dtype %d", dtype);
+    }
+    return fllm_check_launch("experts_down");
+}

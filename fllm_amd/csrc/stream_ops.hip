@@ -94,7 +94,64 @@ stream_add_kernel(float *__restrict__ x, const int32_t *__restrict__ ids, const 
     }
 }
 
+// A branch that is normed on its way into the stream: v = sum of the row's `parts` partial branches (in index order),
+// x[r] += v * rsqrt(mean(v^2) + eps) * gain (normalize 0: x[r] += v * gain).  `gain` is whatever multiplies the normed
+// branch lane by lane: the norm's weight, a layer scale and the constant of the residual sum in one vector.  With
+// `next_w`, the RMSNorm of the new row (its own eps) is written to `next_out` as well, the norm that reads the stream
+// next.  One workgroup a row, sums in a fixed order: a row gives the same bits whatever else is in the batch.
+template <typename B, typename T>
+__global__ void __launch_bounds__(kBlock)
+postnorm_add_kernel(float *__restrict__ x, const B *__restrict__ branch, int parts, const float *__restrict__ gain, float eps,
+                    int normalize, const float *__restrict__ next_w, float next_eps, T *__restrict__ next_out, int width) {
+    __shared__ float scratch[kWaves];
+    const size_t r = blockIdx.x;
+    const B *src = branch + r * parts * width;
+    float *dst = x + r * width;
+    auto value = [&](int c) {
+        float v = to_f32<B>(src[c]);
+        for (int k = 1; k < parts; k++) v += to_f32<B>(src[(size_t)k * width + c]);
+        return v;
+    };
+    float inv = 1.0f;
+    if (normalize) {
+        float ss = 0.f;
+        for (int c = threadIdx.x; c < width; c += kBlock) {
+            const float v = value(c);
+            ss += v * v;
+        }
+        ss = block_sum<kWaves>(ss, scratch);
+        inv = 1.0f / sqrtf(ss / (float)width + eps);
+    }
+    float ss2 = 0.f;
+    for (int c = threadIdx.x; c < width; c += kBlock) {
+        const float v = dst[c] + value(c) * inv * gain[c];
+        dst[c] = v;
+        ss2 += v * v;
+    }
+    if (next_w == nullptr) return;
+    ss2 = block_sum<kWaves>(ss2, scratch);
+    const float inv2 = 1.0f / sqrtf(ss2 / (float)width + next_eps);
+    for (int c = threadIdx.x; c < width; c += kBlock) next_out[r * width + c] = from_f32<T>(dst[c] * inv2 * next_w[c]);   // the thread's own stores
+}
+
 }  // namespace
+
+extern "C" int fllm_postnorm_add(float *x, const void *branch, int branch_dtype, int parts, const float *gain, float eps, int normalize,
+                                 const float *next_w, float next_eps, void *next_out, int next_dtype, int rows, int width,
+                                 hipStream_t stream) {
+    FLLM_REQUIRE(rows >= 0 && width > 0 && parts > 0, "postnorm_add: bad sizes");
+    FLLM_REQUIRE(x && branch && gain && ((next_w == nullptr) == (next_out == nullptr)), "postnorm_add: operands missing");
+    if (rows == 0) return 0;
+#define FLLM_POSTNORM(B, T) hipLaunchKernelGGL((postnorm_add_kernel<B, T>), dim3(rows), dim3(kBlock), 0, stream, x, (const B *)branch, \
+                                               parts, gain, eps, normalize, next_w, next_eps, (T *)next_out, width)
+    if (branch_dtype == FLLM_F32 && next_dtype == FLLM_F32) FLLM_POSTNORM(float, float);
+    else if (branch_dtype == FLLM_F32 && next_dtype == FLLM_BF16) FLLM_POSTNORM(float, bf16_t);
+    else if (branch_dtype == FLLM_BF16 && next_dtype == FLLM_F32) FLLM_POSTNORM(bf16_t, float);
+    else if (branch_dtype == FLLM_BF16 && next_dtype == FLLM_BF16) FLLM_POSTNORM(bf16_t, bf16_t);
+    else FLLM_REQUIRE(false, "postnorm_add: unknown dtypes %d, %d", branch_dtype, next_dtype);
+#undef FLLM_POSTNORM
+    return fllm_check_launch("postnorm_add");
+}
 
 extern "C" int fllm_rmsnorm_pair(const float *x, const float *w1, const float *w2, void *out1, void *out2, int rows, int width,
                                  float eps1, float eps2, int out_dtype, hipStream_t stream) {

@@ -49,7 +49,7 @@ assert SAMPLE_ROW_BYTES == 32
 _lib = None
 
 
-ABI_VERSION = 12
+ABI_VERSION = 13
 
 
 def load_library(build_if_missing: bool = True):
@@ -80,9 +80,15 @@ def load_library(build_if_missing: bool = True):
         "fllm_add_residual": [c_void, c_void, c_int, c_int, c_int, c_void],
         "fllm_add_rmsnorm": [c_void, c_void, c_int, c_void, c_void, c_int, c_int, c_float, c_int, c_void],
         "fllm_rope_kv_store": [c_void, c_void, c_void, c_void, c_int, c_void, c_void, c_int, c_void, c_void, c_int,
-                               c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void],
+                               c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_void],
         "fllm_attention": [c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_int,
-                           c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_void, c_size, c_void],
+                           c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_int, c_int, c_int, c_void, c_size,
+                           c_void],
+        "fllm_postnorm_add": [c_void, c_void, c_int, c_int, c_void, c_float, c_int, c_void, c_float, c_void, c_int, c_int, c_int, c_void],
+        "fllm_route_topk": [c_void, c_int, c_void, c_int, c_int, c_int, c_int, c_void, c_void, c_int, c_void],
+        "fllm_experts_gate_up": [c_void, c_int, c_void, c_void, c_int, c_int, c_void, c_int, c_int, c_int, c_void, c_float, c_float,
+                                 c_float, c_int, c_void],
+        "fllm_experts_down": [c_void, c_void, c_int, c_void, c_int, c_int, c_int, c_void, c_int, c_void],
         "fllm_attention_sloped": [c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_int,
                                   c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void, c_void],
         "fllm_norm_linear": [c_void, c_void, c_float, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
@@ -632,9 +638,12 @@ class Ops:
     def rope_kv_store(self, qkv: torch.Tensor, row_pos: torch.Tensor, row_seg: torch.Tensor, tables: torch.Tensor,
                       cos: torch.Tensor, sin: torch.Tensor, k_pages: Optional[torch.Tensor],
                       v_pages: Optional[torch.Tensor], heads: int, kv_heads: int, head_dim: int, rope_dims: int,
-                      pairing: int, page_size: int) -> None:
+                      pairing: int, page_size: int, v_dim: Optional[int] = None, key_chunk: int = 8) -> None:
+        """`v_dim`: lanes of a value head where they differ from the keys'; `key_chunk`: values of a key that lie together
+        in a page (8; 1 for head sizes that are no multiple of 8)."""
         rows = qkv.shape[0]
-        _dense(qkv, "qkv", None, (rows, (heads + 2 * kv_heads) * head_dim))
+        v_dim = head_dim if v_dim is None else int(v_dim)
+        _dense(qkv, "qkv", None, (rows, (heads + kv_heads) * head_dim + kv_heads * v_dim))
         _need(qkv.dtype in _DTYPE_CODE, f"dtype {qkv.dtype} unsupported")
         _dense(row_pos, "row_pos", torch.int32, (rows,))
         _dense(row_seg, "row_seg", torch.int32, (rows,))
@@ -646,15 +655,15 @@ class Ops:
         _need(cos.dim() == 2 and cos.shape[1] == half, f"rotary tables must be [positions, {half}]")
         store = k_pages is not None
         num_pages = 0
-        _need(head_dim % 8 == 0, f"head size {head_dim}: keys are stored in chunks of 8 values")
+        _need(key_chunk > 0 and head_dim % key_chunk == 0, f"head size {head_dim}: keys cannot be stored in chunks of {key_chunk} values")
         if store:
             num_pages = k_pages.shape[0]
-            _dense(k_pages, "k_pages", qkv.dtype, (num_pages, kv_heads, head_dim // 8, page_size, 8))
-            _dense(v_pages, "v_pages", qkv.dtype, (num_pages, kv_heads, head_dim, page_size))
+            _dense(k_pages, "k_pages", qkv.dtype, (num_pages, kv_heads, head_dim // key_chunk, page_size, key_chunk))
+            _dense(v_pages, "v_pages", qkv.dtype, (num_pages, kv_heads, v_dim, page_size))
         self._check(self.lib.fllm_rope_kv_store(
             _ptr(qkv), _ptr(row_pos), _ptr(row_seg), _ptr(tables), tables.shape[1], _ptr(cos), _ptr(sin), cos.shape[0],
-            _ptr(k_pages), _ptr(v_pages), num_pages, rows, heads, kv_heads, head_dim, rope_dims, pairing, page_size,
-            _DTYPE_CODE[qkv.dtype], 1 if store else 0, self._stream()))
+            _ptr(k_pages), _ptr(v_pages), num_pages, rows, heads, kv_heads, head_dim, v_dim, rope_dims, pairing, page_size,
+            key_chunk, _DTYPE_CODE[qkv.dtype], 1 if store else 0, self._stream()))
 
     def attention_workspace_bytes(self, rows: int, heads: int, kv_heads: int, head_dim: int, max_context: int) -> int:
         return int(self.lib.fllm_attention_workspace_bytes(rows, heads, kv_heads, head_dim, max_context))
@@ -663,19 +672,26 @@ class Ops:
                   row_pos: torch.Tensor, row_seg: torch.Tensor, seg_start: torch.Tensor, out: torch.Tensor, heads: int, kv_heads: int,
                   head_dim: int, page_size: int, scale: float, window: Optional[int], max_context: int,
                   uniform_rows: int = 0, workspace: Optional[torch.Tensor] = None, single_from: Optional[int] = None,
-                  head_slopes: Optional[torch.Tensor] = None) -> torch.Tensor:
+                  head_slopes: Optional[torch.Tensor] = None, v_dim: Optional[int] = None, chunk: Optional[int] = None,
+                  key_chunk: int = 8) -> torch.Tensor:
         """`q` may be a column slice of a wider row-major matrix (the fused qkv buffer).
         `max_context` bounds pos + 1 over the rows; the segments from `single_from` on have one row each
         (`uniform_rows` = 1 is `single_from` = 0: a decode step; by default no segment is known to).
         `head_slopes` (float32 [heads]): every score gets head_slopes[head] * (key position - row position) added, for
-        position encodings that bias scores; such a call runs the plain kernel in both precisions."""
+        position encodings that bias scores; such a call runs the plain kernel in both precisions.
+        `v_dim`: lanes of a value head where they differ from the keys' (`out` is [rows, heads * v_dim]); `chunk`: a row sees
+        no key before the start of its own chunk of that many positions (chunks counted from position 0); `key_chunk`: values
+        of a key that lie together in a page.  The matrix-core kernels take v_dim == head_dim and key chunks of 8."""
         rows = q.shape[0]
+        v_dim = head_dim if v_dim is None else int(v_dim)
+        chunk = int(chunk) if chunk else 0
+        _need(chunk >= 0 and key_chunk > 0 and head_dim % key_chunk == 0, "attention: bad chunk of positions or of key values")
         _need(q.is_cuda and q.dim() == 2 and q.stride(1) == 1 and q.shape[1] == heads * head_dim,
               f"q must be [rows, {heads * head_dim}] with unit column stride")
         _need(q.dtype in _DTYPE_CODE, f"dtype {q.dtype} unsupported")
         num_pages = k_pages.shape[0]
-        _dense(k_pages, "k_pages", q.dtype, (num_pages, kv_heads, head_dim // 8, page_size, 8))
-        _dense(v_pages, "v_pages", q.dtype, (num_pages, kv_heads, head_dim, page_size))
+        _dense(k_pages, "k_pages", q.dtype, (num_pages, kv_heads, head_dim // key_chunk, page_size, key_chunk))
+        _dense(v_pages, "v_pages", q.dtype, (num_pages, kv_heads, v_dim, page_size))
         _dense(tables, "tables", torch.int32)
         _need(tables.dim() == 2, "tables must be [segments, pages]")
         _dense(row_pos, "row_pos", torch.int32, (rows,))
@@ -683,7 +699,7 @@ class Ops:
         _dense(seg_start, "seg_start", torch.int32)
         _need(seg_start.numel() >= 2, "seg_start must hold at least one segment")
         _need(tables.shape[0] >= seg_start.numel() - 1, "tables must have a row per segment")
-        _dense(out, "out", q.dtype, (rows, heads * head_dim))
+        _dense(out, "out", q.dtype, (rows, heads * v_dim))
         ws_ptr, ws_bytes = None, 0
         if workspace is not None:
             _need(workspace.is_cuda and workspace.is_contiguous(), "workspace must be a dense GPU tensor")
@@ -691,6 +707,7 @@ class Ops:
         q_stride = q.stride(0) if rows > 1 else heads * head_dim
         num_segs = seg_start.numel() - 1
         if head_slopes is not None:
+            _need(v_dim == head_dim and not chunk and key_chunk == 8, "biased scores come with one width of keys and values and no chunks")
             _dense(head_slopes, "head_slopes", torch.float32, (heads,))
             self._check(self.lib.fllm_attention_sloped(
                 _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(tables), tables.shape[1], _ptr(row_pos), _ptr(row_seg),
@@ -702,9 +719,9 @@ class Ops:
         _need(0 <= single_from <= num_segs and num_segs - single_from <= rows, f"single_from {single_from} does not fit {num_segs} segments of {rows} rows")
         self._check(self.lib.fllm_attention(
             _ptr(q), q_stride, _ptr(k_pages), _ptr(v_pages), _ptr(tables), tables.shape[1], _ptr(row_pos), _ptr(row_seg),
-            _ptr(seg_start), seg_start.numel() - 1, _ptr(out), rows, heads, kv_heads, head_dim, page_size, num_pages, float(scale),
-            int(window) if window else 0, _DTYPE_CODE[q.dtype], int(max_context), int(single_from), ws_ptr, ws_bytes,
-            self._stream()))
+            _ptr(seg_start), seg_start.numel() - 1, _ptr(out), rows, heads, kv_heads, head_dim, v_dim, page_size, num_pages,
+            float(scale), int(window) if window else 0, chunk, key_chunk, _DTYPE_CODE[q.dtype], int(max_context), int(single_from),
+            ws_ptr, ws_bytes, self._stream()))
         return out
 
     # ---- parts of other layer designs ----------------------------------------------------------------------
@@ -760,6 +777,73 @@ class Ops:
         self._check(self.lib.fllm_stream_add(_ptr(x), _ptr(ids) if table is not None else None, _ptr(table), code, vocab,
                                              float(scale), _ptr(vec), rows, width, self._stream()))
         return x
+
+    def postnorm_add(self, x: torch.Tensor, branch: torch.Tensor, gain: torch.Tensor, eps: Optional[float], parts: int = 1,
+                     next_weight: Optional[torch.Tensor] = None, next_eps: float = 0.0,
+                     next_out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """x[r] += v * rsqrt(mean(v^2) + eps) * gain with v = the sum of the row's `parts` partial branches (`branch` is
+        [rows * parts, width], a row's parts one after the other); eps None: x[r] += v * gain.  With `next_weight`, the
+        RMSNorm of the new rows (`next_eps`) goes to `next_out`."""
+        rows, width = x.shape
+        _dense(x, "x", torch.float32)
+        _dense(branch, "branch", None, (rows * parts, width))
+        _need(branch.dtype in _DTYPE_CODE, f"branch dtype {branch.dtype} unsupported")
+        _dense(gain, "gain", torch.float32, (width,))
+        _need((next_weight is None) == (next_out is None), "the norm behind the sum needs a weight and an output")
+        code = F32
+        if next_weight is not None:
+            _dense(next_weight, "next_weight", torch.float32, (width,))
+            _dense(next_out, "next_out", None, (rows, width))
+            _need(next_out.dtype in _DTYPE_CODE, f"next_out dtype {next_out.dtype} unsupported")
+            code = _DTYPE_CODE[next_out.dtype]
+        self._check(self.lib.fllm_postnorm_add(_ptr(x), _ptr(branch), _DTYPE_CODE[branch.dtype], int(parts), _ptr(gain),
+                                               float(eps or 0.0), 0 if eps is None else 1, _ptr(next_weight), float(next_eps),
+                                               _ptr(next_out), code, rows, width, self._stream()))
+        return x
+
+    def route_topk(self, h: torch.Tensor, w_router: torch.Tensor, top: int, ids: torch.Tensor, weights: torch.Tensor):
+        """score = sigmoid(h @ w_router.T) in float32; ids[r, k] / weights[r, k]: the expert with the k-th largest score of
+        row r (the lower index among equals) and that score."""
+        rows, K = h.shape
+        E = w_router.shape[0]
+        _need(h.is_cuda and h.dim() == 2 and h.stride(1) == 1 and h.dtype in _DTYPE_CODE, "h must be a row-major GPU matrix")
+        _dense(w_router, "w_router", h.dtype, (E, K))
+        _dense(ids, "ids", torch.int32, (rows, top))
+        _dense(weights, "weights", torch.float32, (rows, top))
+        self._check(self.lib.fllm_route_topk(_ptr(h), h.stride(0) if rows > 1 else K, _ptr(w_router), rows, K, E, int(top), _ptr(ids),
+                                             _ptr(weights), _DTYPE_CODE[h.dtype], self._stream()))
+        return ids, weights
+
+    def experts_gate_up(self, h: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gate_up: torch.Tensor, act: torch.Tensor,
+                        limit: float = 0.0, alpha: float = 1.0, up_offset: float = 0.0) -> torch.Tensor:
+        """act[r * top + k] = a(g) * (u + up_offset), g and u the gate and up rows of expert ids[r, k] times (h[r] *
+        weights[r, k]); w_gate_up [experts, 2 * inter, width] (gate rows, then up rows); the activation as in `glu_clamped`."""
+        rows, K = h.shape
+        top = ids.shape[1]
+        E, two_i = w_gate_up.shape[0], w_gate_up.shape[1]
+        _need(h.is_cuda and h.dim() == 2 and h.stride(1) == 1 and h.dtype in _DTYPE_CODE, "h must be a row-major GPU matrix")
+        _dense(w_gate_up, "w_gate_up", h.dtype, (E, two_i, K))
+        _need(two_i % 2 == 0, "w_gate_up holds gate rows and as many up rows")
+        _dense(ids, "ids", torch.int32, (rows, top))
+        _dense(weights, "weights", torch.float32, (rows, top))
+        _dense(act, "act", h.dtype, (rows * top, two_i // 2))
+        self._check(self.lib.fllm_experts_gate_up(_ptr(h), h.stride(0) if rows > 1 else K, _ptr(ids), _ptr(weights), rows, top,
+                                                  _ptr(w_gate_up), E, two_i // 2, K, _ptr(act), float(limit), float(alpha),
+                                                  float(up_offset), _DTYPE_CODE[h.dtype], self._stream()))
+        return act
+
+    def experts_down(self, act: torch.Tensor, ids: torch.Tensor, w_down: torch.Tensor, out: torch.Tensor) -> torch.Tensor:
+        """out[p] = w_down[ids[p]] @ act[p] for every (row, pick) pair p, float32; w_down [experts, width, inter]."""
+        pairs, inter = act.shape
+        E, N = w_down.shape[0], w_down.shape[1]
+        _dense(act, "act")
+        _need(act.dtype in _DTYPE_CODE, f"dtype {act.dtype} unsupported")
+        _dense(w_down, "w_down", act.dtype, (E, N, inter))
+        _need(ids.is_cuda and ids.is_contiguous() and ids.dtype == torch.int32 and ids.numel() == pairs, "ids must name an expert a pair")
+        _dense(out, "out", torch.float32, (pairs, N))
+        self._check(self.lib.fllm_experts_down(_ptr(act), _ptr(ids), pairs, _ptr(w_down), E, N, inter, _ptr(out),
+                                               _DTYPE_CODE[act.dtype], self._stream()))
+        return out
 
     def _talking_pages(self, k_pages, v_pages, dtype, kv_heads, k_dim, v_dim, page_size, key_chunk):
         _need(key_chunk > 0 and k_dim % key_chunk == 0, f"keys of {k_dim} values cannot lie in chunks of {key_chunk}")

@@ -2,8 +2,10 @@
 
 q, k, v = one product with the concatenated projection matrix; rotary on q and k; k and v stored
 in the pages of the row's request; every row attends to the keys of its request at positions
-[pos - window + 1, pos] (all from 0 without a window), heads grouped over the key/value heads
-(h -> h / (heads / kv_heads)); output projection added to the residual stream
+[pos - window + 1, pos] (all from 0 without a window) and, with `chunk`, to none before the start of its
+own chunk of that many positions (chunks counted from the request's first position), heads grouped over
+the key/value heads (h -> h / (heads / kv_heads)); values may have a width of their own (`value_head_dim`);
+output projection added to the residual stream, or stored as a branch for a block that norms it first
 (rust/engine/src/rust_decoder.rs:8827-8835 projections, :8895-8898 rotary, :8955-8963 cache write,
 :6065-6166 scores, mask, softmax and output, :9025 and :9059 projection and residual).
 """
@@ -18,15 +20,17 @@ from .base import INIT_BIAS, INIT_MATRIX, KVNeed, Mixer, add_and_prepare, fused_
 
 class PagedAttention(Mixer):
     graph_safe = True      # forward launches kernels only: no per-step decision on the host
+    stores_branch = True   # forward(..., branch=t) stores the output projection in t instead of adding it to the stream
     KEY_CHUNK = 8          # values of a key that lie together in a page (csrc/common.h, key_offset)
 
     @classmethod
     def tensor_shapes(cls, spec):
         h, nh, nkv, d = spec["hidden_size"], spec["num_heads"], spec["num_kv_heads"], spec["head_dim"]
+        dv = spec.get("value_head_dim") or d
         return {
-            "q": ((nh * d, h), INIT_MATRIX), "k": ((nkv * d, h), INIT_MATRIX), "v": ((nkv * d, h), INIT_MATRIX),
-            "o": ((h, nh * d), INIT_MATRIX),
-            "q_bias": ((nh * d,), INIT_BIAS), "k_bias": ((nkv * d,), INIT_BIAS), "v_bias": ((nkv * d,), INIT_BIAS),
+            "q": ((nh * d, h), INIT_MATRIX), "k": ((nkv * d, h), INIT_MATRIX), "v": ((nkv * dv, h), INIT_MATRIX),
+            "o": ((h, nh * dv), INIT_MATRIX),
+            "q_bias": ((nh * d,), INIT_BIAS), "k_bias": ((nkv * d,), INIT_BIAS), "v_bias": ((nkv * dv,), INIT_BIAS),
             "o_bias": ((h,), INIT_BIAS),
         }
 
@@ -38,16 +42,24 @@ class PagedAttention(Mixer):
         self.head_dim = int(spec["head_dim"])
         self.scale = float(spec["scale"])
         self.window = spec.get("window")
+        self.chunk = spec.get("chunk")
+        self.v_dim = int(spec.get("value_head_dim") or self.head_dim)
         if self.heads % self.kv_heads != 0:
             raise ValueError(f"head count {self.heads} is not a multiple of key/value head count {self.kv_heads}")
         if self.window is not None and self.window <= 0:
             raise ValueError("an attention window must be positive")
-        if self.head_dim % self.KEY_CHUNK != 0:
-            raise ValueError(f"head size {self.head_dim}: the attention kernels store keys in chunks of {self.KEY_CHUNK} values, "
-                             f"head sizes come in steps of {self.KEY_CHUNK}")
-        if spec.get("value_head_dim") not in (None, self.head_dim):
-            raise ValueError(f"this attention's kernels read keys and values of one width: values of "
-                             f"{spec.get('value_head_dim')} beside keys of {self.head_dim} need a mixer of their own")
+        if self.chunk is not None and self.chunk <= 0:
+            raise ValueError("a chunk of positions must be positive")
+        # keys lie in chunks of 8 values inside a page where the head size allows it (what the matrix-core kernels read);
+        # other head sizes store a head's lanes one by one and run the plain kernels
+        self.key_chunk = self.KEY_CHUNK if self.head_dim % self.KEY_CHUNK == 0 else 1
+        # what only the plain kernels take (values of another width than the keys, a chunk of positions in the fused
+        # store, key lanes one by one): named once, so that every call hands over the same arguments
+        self.shape_args = {}
+        if self.v_dim != self.head_dim:
+            self.shape_args["v_dim"] = self.v_dim
+        if self.key_chunk != self.KEY_CHUNK:
+            self.shape_args["key_chunk"] = self.key_chunk
         position = spec.get("position")
         self.position = None
         if position is not None:
@@ -77,7 +89,7 @@ class PagedAttention(Mixer):
                   None if weights.get("v_bias") is None else rt.vector(weights["v_bias"])]
         self.b_qkv = None
         if any(b is not None for b in biases):
-            sizes = (self.heads * self.head_dim, self.kv_heads * self.head_dim, self.kv_heads * self.head_dim)
+            sizes = (self.heads * self.head_dim, self.kv_heads * self.head_dim, self.kv_heads * self.v_dim)
             self.b_qkv = torch.cat([b if b is not None else torch.zeros(n, dtype=torch.float32, device=rt.device)
                                     for b, n in zip(biases, sizes)]).contiguous()
         self.b_o = rt.vector(weights["o_bias"]) if weights.get("o_bias") is not None else None
@@ -93,14 +105,15 @@ class PagedAttention(Mixer):
         return torch.tensor([h * head_dim + j for h in range(heads) for j in one], dtype=torch.long)
 
     def cache_need(self):
-        # keys and values of one width, keys in chunks of 8 values (16 bytes in bfloat16): what the kernels take
-        return KVNeed(self.kv_heads, self.head_dim, self.head_dim, self.window, key_chunk=self.KEY_CHUNK)
+        # keys in chunks of 8 values (16 bytes in bfloat16) where the head size allows it.  A chunk of positions is a mask,
+        # not a window: earlier chunks keep their pages until the request ends.
+        return KVNeed(self.kv_heads, self.head_dim, self.v_dim, self.window, key_chunk=self.key_chunk)
 
     def forward(self, ctx, h, residual, binding, branch=None):
         rt, ops = self.rt, self.rt.ops
         rows = h.shape[0]
         nh, nkv, d = self.heads, self.kv_heads, self.head_dim
-        qkv = rt.empty((rows, (nh + 2 * nkv) * d))
+        qkv = rt.empty((rows, (nh + nkv) * d + nkv * self.v_dim))
         ops.linear(h, self.w_qkv, qkv, bias=self.b_qkv)
         tables = ctx.tables[binding.group]
         if self.position is not None:
@@ -109,10 +122,10 @@ class PagedAttention(Mixer):
             cos, sin, dims, pairing = ctx.no_rotation(rt)
         ops.rope_kv_store(qkv, ctx.row_pos, ctx.row_seg, tables, cos, sin,
                           binding.k_pages if binding.writes else None, binding.v_pages if binding.writes else None,
-                          nh, nkv, d, dims, pairing, binding.page_size)
+                          nh, nkv, d, dims, pairing, binding.page_size, **self.shape_args)
         self._attend_and_project(ctx, qkv[:, : nh * d], residual, binding, branch=branch)
 
-    def forward_from_residual(self, ctx, residual, norm, binding) -> bool:
+    def forward_from_residual(self, ctx, residual, norm, binding, branch=None) -> bool:
         """Decode-sized steps in bfloat16: the norm before the mixer, the q/k/v product, rotary and the
         cache store are one kernel.  False: not taken, the block runs norm and `forward`."""
         rt, ops = self.rt, self.rt.ops
@@ -121,6 +134,8 @@ class PagedAttention(Mixer):
         form = fused_form(ops, rows, self.hidden, self.w_qkv) if hasattr(ops, "norm_qkv_rope_store") else None
         if rt.dtype != torch.bfloat16 or self.pairing != 1 or prologue is None or form is None or self.head_dim % 4 != 0:
             return False
+        if self.shape_args:
+            return False         # the fused store takes keys and values of one width, keys in chunks of 8
         norm_scale, norm_eps = prologue
         nh, nkv, d = self.heads, self.kv_heads, self.head_dim
         if self.position is not None:
@@ -135,7 +150,7 @@ class PagedAttention(Mixer):
                                 ctx.tables[binding.group], cos, sin, binding.k_pages if binding.writes else None,
                                 binding.v_pages if binding.writes else None, nh, nkv, d, dims, binding.page_size,
                                 bias=self.b_qkv, **({"prepared": prepared} if prepared is not None else {}))
-        self._attend_and_project(ctx, q, residual, binding)
+        self._attend_and_project(ctx, q, residual, binding, branch=branch)
         return True
 
     def forward_branch(self, ctx, h, binding):
@@ -158,7 +173,8 @@ class PagedAttention(Mixer):
         rows = q.shape[0]
         nh, nkv, d = self.heads, self.kv_heads, self.head_dim
         tables = ctx.tables[binding.group]
-        out = rt.empty((rows, nh * d))
+        out = rt.empty((rows, nh * self.v_dim))
+        shape_args = dict(self.shape_args, chunk=self.chunk) if self.chunk else self.shape_args
         # Single rows behind portions of prompts: with long contexts they go to the kernel that splits a context over
         # workgroups (a second launch); with short ones they ride along in the portions' launch, which is faster then.
         single_from = ctx.single_rows_from()
@@ -167,12 +183,13 @@ class PagedAttention(Mixer):
         slopes = getattr(self.position, "score_slopes", None)      # a position encoding may bias scores by distance
         if slopes is not None:
             ops.attention(q, binding.k_pages, binding.v_pages, tables, ctx.row_pos, ctx.row_seg, ctx.seg_start,
-                          out, nh, nkv, d, binding.page_size, self.scale, self.window, ctx.max_context, head_slopes=slopes)
+                          out, nh, nkv, d, binding.page_size, self.scale, self.window, ctx.max_context, head_slopes=slopes,
+                          **shape_args)
         else:
             ops.attention(q, binding.k_pages, binding.v_pages, tables, ctx.row_pos, ctx.row_seg, ctx.seg_start,
                           out, nh, nkv, d, binding.page_size, self.scale, self.window, ctx.max_context,
                           single_from=single_from,
-                          workspace=ctx.attention_workspace(rt, rows, nh, nkv, d))
+                          workspace=ctx.attention_workspace(rt, rows, nh, nkv, d), **shape_args)
         if branch is not None:
             ops.linear(out, self.w_o, branch, bias=self.b_o)
         elif not add_and_prepare(ctx, ops, out, self.w_o, residual, self.b_o):

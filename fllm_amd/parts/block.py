@@ -1,10 +1,14 @@
 """Arrangement of parts in a layer.  `prenorm`: x += mixer(norm(x)); x += feed_forward(norm(x))
 (rust/engine/src/rust_decoder.rs:8764-8766, :9059-9088).  `parallel`: x += mixer(norm_a(x)) + feed_forward(norm_b(x)),
-both branches behind norms of their own of the same x."""
+both branches behind norms of their own of the same x.  `sandwich`: a norm before and a norm behind each part,
+x += m * s_a * norm_a'(mixer(norm_a(x))); x += m * s_b * norm_b'(feed_forward(norm_b(x))), with a constant m and
+learned vectors s (a scale a lane of each branch)."""
 from __future__ import annotations
 
+import torch
+
 from ..registry import register_part
-from .base import Block
+from .base import INIT_NORM, Block
 
 
 class PreNormBlock(Block):
@@ -135,5 +139,98 @@ class ParallelBlock(Block):
             self.feed_forward.forward(ctx, h_ff, residual)
 
 
+class SandwichBlock(Block):
+    """x += gain_a * rms'(mixer(norm_a x)); x += gain_b * rms'(feed_forward(norm_b x)): every branch is normed again
+    (RMS over its own lanes) before it joins the stream.  gain = residual_mult * layer scale * the second norm's weight,
+    one float32 vector a branch, made once: the kernel that adds a branch norms it on the way (`postnorm_add`).  The
+    norms behind the parts are `mixer_out` and `feed_forward_out` (absent: the branch is scaled and added as it is); the
+    layer scales are the block's own tensors `mixer_scale` and `feed_forward_scale` (optional).
+
+    A part with `stores_branch` writes its output (float32) where the block tells it to (`branch=`); any other part adds
+    into a zeroed buffer that stands in for the stream.  A part may leave several partial rows a token (`branch_parts`),
+    which the adding kernel sums first."""
+
+    @classmethod
+    def tensor_shapes(cls, spec):
+        return {"mixer_scale": ((spec["size"],), INIT_NORM), "feed_forward_scale": ((spec["size"],), INIT_NORM)}
+
+    def __init__(self, spec, weights, rt, mixer=None, feed_forward=None, norms=None):
+        super().__init__(spec, weights, rt)
+        self.mixer = mixer
+        self.feed_forward = feed_forward
+        self.size = int(spec["size"])
+        self.mixer_norm = norms["mixer"]
+        self.feed_forward_norm = norms["feed_forward"] if feed_forward is not None else None
+        mult = float(spec.get("residual_mult", 1.0))
+        self.mixer_gain, self.mixer_eps = self._gain(mult, weights.get("mixer_scale"), norms.get("mixer_out"))
+        if feed_forward is not None:
+            self.feed_forward_gain, self.feed_forward_eps = self._gain(mult, weights.get("feed_forward_scale"),
+                                                                       norms.get("feed_forward_out"))
+
+    def _gain(self, mult, scale, out_norm):
+        """(gain vector, eps of the norm behind the part or None when there is none)."""
+        gain = torch.full((self.size,), mult, dtype=torch.float32, device=self.rt.device)
+        eps = None
+        if out_norm is not None:
+            prologue = getattr(out_norm, "fused_prologue", lambda: None)()
+            if prologue is None:
+                raise ValueError("the norm behind a part must be of the form x * rsqrt(mean x^2 + eps) * weight")
+            gain = gain * prologue[0]
+            eps = float(prologue[1])
+        if scale is not None:
+            gain = gain * self.rt.vector(scale)
+        return gain.contiguous(), eps
+
+    def first_norm(self):
+        return None          # this block's first norm rides on the sum before it only inside the block itself
+
+    def _branch(self, part, rows):
+        return self.rt.empty((rows * int(getattr(part, "branch_parts", 1)), self.size), torch.float32)
+
+    def forward(self, ctx, residual, binding):
+        rt, ops = self.rt, self.rt.ops
+        rows = residual.shape[0]
+        ctx.then_norm = ctx.prepared = None          # no sum of this block's parts is read by a norm the parts know
+        # ---- mixer
+        mixer = self.mixer
+        if getattr(mixer, "stores_branch", False):
+            branch = self._branch(mixer, rows)
+            fused = getattr(mixer, "forward_from_residual", None)
+            if fused is None or not fused(ctx, residual, self.mixer_norm, binding, branch=branch):
+                mixer.forward(ctx, self.mixer_norm.forward(ctx, residual), None, binding, branch=branch)
+        else:
+            branch = torch.zeros((rows, self.size), dtype=torch.float32, device=rt.device)
+            mixer.forward(ctx, self.mixer_norm.forward(ctx, residual), branch, binding)
+        ff = self.feed_forward
+        if ff is None:
+            ops.postnorm_add(residual, branch, self.mixer_gain, self.mixer_eps, parts=branch.shape[0] // rows)
+            return
+        # the sum of the mixer's branch and the norm before the feed-forward are one pass over the row, unless the
+        # feed-forward reads the stream through its norm itself
+        begin = getattr(ff, "begin_from_residual", None) if getattr(ff, "stores_branch", False) else None
+        prologue = getattr(self.feed_forward_norm, "fused_prologue", lambda: None)()
+        takes_stream = begin is not None and getattr(ff, "begins_from_residual", lambda rows: False)(rows)
+        h = None
+        if prologue is not None and not takes_stream:
+            h = rt.empty((rows, self.size))
+            ops.postnorm_add(residual, branch, self.mixer_gain, self.mixer_eps, parts=branch.shape[0] // rows,
+                             next_weight=prologue[0], next_eps=prologue[1], next_out=h)
+        else:
+            ops.postnorm_add(residual, branch, self.mixer_gain, self.mixer_eps, parts=branch.shape[0] // rows)
+        # ---- feed-forward
+        if getattr(ff, "stores_branch", False):
+            branch = self._branch(ff, rows)
+            begun = begin(ctx, residual, self.feed_forward_norm) if takes_stream else None
+            if begun is not None:
+                ff.finish(ctx, begun, None, branch=branch)
+            else:
+                ff.forward(ctx, h if h is not None else self.feed_forward_norm.forward(ctx, residual), None, branch=branch)
+        else:
+            branch = torch.zeros((rows, self.size), dtype=torch.float32, device=rt.device)
+            ff.forward(ctx, h if h is not None else self.feed_forward_norm.forward(ctx, residual), branch)
+        ops.postnorm_add(residual, branch, self.feed_forward_gain, self.feed_forward_eps, parts=branch.shape[0] // rows)
+
+
 register_part("block", "prenorm", PreNormBlock)
+register_part("block", "sandwich", SandwichBlock)
 register_part("block", "parallel", ParallelBlock)

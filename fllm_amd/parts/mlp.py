@@ -107,6 +107,7 @@ class ClampedGLU(FeedForward):
     """x += W_down (a(g) * (u + up_offset)) with g = min(W_gate n, limit), u = clamp(W_up n, -limit, limit) and
     a(g) = g * sigmoid(alpha * g).  Gate and up are one product with the concatenated matrix."""
     graph_safe = True
+    stores_branch = True   # forward(..., branch=t) stores the down projection in t instead of adding it to the stream
 
     @classmethod
     def tensor_shapes(cls, spec):
@@ -125,6 +126,13 @@ class ClampedGLU(FeedForward):
         rt.tile_for_decode(self.w_down)
         rt.tile_for_decode(self.w_gate_up, gate_up=True, priority=1)
 
+    def begins_from_residual(self, rows: int) -> bool:
+        """Whether `begin_from_residual` would take a step of `rows` rows (an arrangement that can fold this part's
+        norm into another kernel asks first)."""
+        ops = self.rt.ops
+        return (self.rt.dtype == torch.bfloat16 and hasattr(ops, "norm_gate_up_glu")
+                and fused_form(ops, rows, self.hidden, self.w_gate_up, gate_up=True) == "resident")
+
     def begin_from_residual(self, ctx, residual, norm):
         """Decode-sized steps in bfloat16: the norm before this part, the gate/up product and the activation are one
         kernel that reads the residual stream; the activations come back and `finish` adds the down projection, which
@@ -140,10 +148,13 @@ class ClampedGLU(FeedForward):
         ops.norm_gate_up_glu(residual, prologue[0], prologue[1], self.w_gate_up, act, self.limit, self.alpha, self.up_offset)
         return act
 
-    def finish(self, ctx, act, residual):
-        self.rt.ops.linear(act, self.w_down, residual, accumulate=True)
+    def finish(self, ctx, act, residual, branch=None):
+        if branch is not None:
+            self.rt.ops.linear(act, self.w_down, branch)
+        else:
+            self.rt.ops.linear(act, self.w_down, residual, accumulate=True)
 
-    def forward(self, ctx, h, residual):
+    def forward(self, ctx, h, residual, branch=None):
         rt, ops = self.rt, self.rt.ops
         rows = h.shape[0]
         act = rt.empty((rows, self.inter))
@@ -158,7 +169,7 @@ class ClampedGLU(FeedForward):
             gate_up = rt.empty((rows, 2 * self.inter))
             ops.linear(h, self.w_gate_up, gate_up)
             ops.glu_clamped(gate_up, act, self.limit, self.alpha, self.up_offset)
-        ops.linear(act, self.w_down, residual, accumulate=True)
+        self.finish(ctx, act, residual, branch)
 
 
 register_part("feed_forward", "gated_mlp", GatedMLP)

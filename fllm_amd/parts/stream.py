@@ -2,7 +2,7 @@
 
 `pass_input`: the input of a pass of looped layers.  x += E[token] * scale for every pass but the first (the output of
 the embedding as the model began with, which the embedding part recomputes from the step's token ids: no copy of it
-is kept), then x += steps[row], one learned vector a pass."""
+is kept), then x += steps[row], one learned vector a pass, where the design has such vectors (`rows` in the spec)."""
 from __future__ import annotations
 
 from ..registry import register_part
@@ -15,21 +15,25 @@ class PassInput(Part):
 
     @classmethod
     def tensor_shapes(cls, spec):
-        return {"steps": ((spec["rows"], spec["size"]), INIT_BIAS)}
+        return {"steps": ((spec["rows"], spec["size"]), INIT_BIAS)} if spec.get("rows") else {}
 
     def __init__(self, spec, weights, rt):
         super().__init__(spec, weights, rt)
-        row, rows = int(spec["row"]), int(spec["rows"])
-        if not 0 <= row < rows:
-            raise ValueError(f"pass {row} of {rows}")
-        self.vector = rt.vector(weights["steps"])[row]        # a view of the shared table: one row, contiguous
+        self.vector = None
+        if spec.get("rows"):
+            row, rows = int(spec["row"]), int(spec["rows"])
+            if not 0 <= row < rows:
+                raise ValueError(f"pass {row} of {rows}")
+            self.vector = rt.vector(weights["steps"])[row]    # a view of the shared table: one row, contiguous
         self.add_embedding = bool(spec.get("add_embedding", False))
+        if self.vector is None and not self.add_embedding:
+            raise ValueError("a pass input that adds nothing")
 
     def forward(self, ctx, x, embedding) -> None:
         """`embedding`: the model's embedding part (its table and scale are what the stream began with)."""
         if self.add_embedding:
             self.rt.ops.stream_add(x, ids=ctx.ids, table=embedding.table, scale=embedding.scale, vec=self.vector)
-        else:
+        elif self.vector is not None:
             self.rt.ops.stream_add(x, vec=self.vector)
 
 

@@ -97,10 +97,12 @@ class ReferenceOps:
         return out
 
     def rope_kv_store(self, qkv, row_pos, row_seg, tables, cos, sin, k_pages, v_pages, heads, kv_heads, head_dim,
-                      rope_dims, pairing, page_size):
+                      rope_dims, pairing, page_size, v_dim=None, key_chunk=8):
         rows = qkv.shape[0]
         half = rope_dims // 2
-        view = qkv.view(rows, heads + 2 * kv_heads, head_dim)
+        v_dim = head_dim if v_dim is None else v_dim
+        rotated = (heads + kv_heads) * head_dim
+        view = qkv[:, :rotated].view(rows, heads + kv_heads, head_dim)
         for r in range(rows):
             seg = int(row_seg[r])
             if seg < 0:
@@ -120,17 +122,19 @@ class ReferenceOps:
                 continue
             page = int(tables[seg, pos // page_size])
             off = pos % page_size
-            # keys lie chunk by chunk in a page: [page][kv_head][head_dim / 8][token][8]
-            k_pages[page, :, :, off, :] = view[r, heads:heads + kv_heads, :].reshape(kv_heads, head_dim // 8, 8)
-            v_pages[page, :, :, off] = view[r, heads + kv_heads:, :]
+            # keys lie chunk by chunk in a page: [page][kv_head][head_dim / key_chunk][token][key_chunk]
+            k_pages[page, :, :, off, :] = view[r, heads:heads + kv_heads, :].reshape(kv_heads, head_dim // key_chunk, key_chunk)
+            v_pages[page, :, :, off] = qkv[r, rotated:].view(kv_heads, v_dim)
 
     def attention_workspace_bytes(self, rows, heads, kv_heads, head_dim, max_context):
         return 0
 
     def attention(self, q, k_pages, v_pages, tables, row_pos, row_seg, seg_start, out, heads, kv_heads, head_dim, page_size, scale,
-                  window, max_context, uniform_rows=0, workspace=None, single_from=None, head_slopes=None):
+                  window, max_context, uniform_rows=0, workspace=None, single_from=None, head_slopes=None, v_dim=None, chunk=None,
+                  key_chunk=8):
         rows = q.shape[0]
         group = heads // kv_heads
+        v_dim = head_dim if v_dim is None else v_dim
         for r in range(rows):
             seg = int(row_seg[r])
             if seg < 0:
@@ -139,6 +143,8 @@ class ReferenceOps:
             pos = int(row_pos[r])
             n = pos + 1
             lo = max(0, n - window) if window else 0
+            if chunk:
+                lo = max(lo, pos - pos % chunk)
             keys = torch.arange(lo, n, device=q.device)
             pages = tables[seg, (keys // page_size).long()].long()
             offs = (keys % page_size).long()
@@ -150,7 +156,44 @@ class ReferenceOps:
                 if head_slopes is not None:
                     s = s + float(head_slopes[h]) * (keys - pos).double()
                 p = torch.softmax(s, dim=0)
-                out[r, h * head_dim:(h + 1) * head_dim] = (p @ v[:, h // group, :]).to(out.dtype)
+                out[r, h * v_dim:(h + 1) * v_dim] = (p @ v[:, h // group, :]).to(out.dtype)
+        return out
+
+    # ---- a branch normed on its way into the stream; routed experts ----
+    def postnorm_add(self, x, branch, gain, eps, parts=1, next_weight=None, next_eps=0.0, next_out=None):
+        rows, width = x.shape
+        v = branch.double().view(rows, parts, width).sum(1)
+        if eps is not None:
+            v = v / torch.sqrt((v * v).mean(-1, keepdim=True) + eps)
+        x.copy_((x.double() + v * gain.double()).to(x.dtype))
+        if next_weight is not None:
+            self.rmsnorm(x, next_weight, next_eps, next_out)
+        return x
+
+    def route_topk(self, h, w_router, top, ids, weights):
+        score = torch.sigmoid((h.double() @ w_router.double().T).float())
+        order = torch.sort(score, dim=1, descending=True, stable=True)[1][:, :top]
+        ids.copy_(order.to(ids.dtype))
+        weights.copy_(torch.gather(score, 1, order))
+        return ids, weights
+
+    def experts_gate_up(self, h, ids, weights, w_gate_up, act, limit=0.0, alpha=1.0, up_offset=0.0):
+        rows, top = ids.shape
+        inter = w_gate_up.shape[1] // 2
+        for r in range(rows):
+            for k in range(top):
+                x = (h[r].float() * weights[r, k]).to(h.dtype).double()
+                y = w_gate_up[int(ids[r, k])].double() @ x
+                g, u = y[:inter], y[inter:]
+                if limit > 0:
+                    g, u = torch.clamp(g, max=limit), torch.clamp(u, -limit, limit)
+                act[r * top + k] = (g / (1.0 + torch.exp(-alpha * g)) * (u + up_offset)).to(act.dtype)
+        return act
+
+    def experts_down(self, act, ids, w_down, out):
+        flat = ids.reshape(-1)
+        for p in range(act.shape[0]):
+            out[p] = (w_down[int(flat[p])].double() @ act[p].double()).to(out.dtype)
         return out
 
     # ---- parts of other layer designs: two norms of one row, clamped gated activation, what a pass of looped layers

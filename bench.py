@@ -226,6 +226,27 @@ def menitar_config(size, layers):
     return cfg, layers
 
 
+DESIGN_EXPERTS, DESIGN_TOP = 8, 2      # routed layers of the Purivik runs: two of eight experts of half the dense width a token
+
+
+def purivik_config(size, layers):
+    """`layers` layers, dense and routed feed-forwards in turn (a token's two experts have the dense layer's lanes between
+    them, so a layer run costs what the dense one costs), of which the middle half runs twice."""
+    mixer = {"heads": size["heads"], "kv_heads": size["kv_heads"], "dim": size["dim"], "vdim": size["dim"],
+             "scale": size["dim"] ** -0.5, "mask": {"size": DESIGN_CHUNK},
+             "rot": {"dims": size["dim"] // 2, "base": 500000.0, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}}
+    dense = {"kind": "dense", "ff": size["ff"], "limit": 7.0}
+    routed = {"kind": "moe", "expert": {"ff": size["ff"] // DESIGN_TOP}, "router": {"experts": DESIGN_EXPERTS, "top": DESIGN_TOP}}
+    cfg = {"architecture": "Purivik", "width": size["width"], "vocab": size["vocab"], "embedding": {"scale": 1.0},
+           "residual_mult": 0.7, "norm": {"eps": 1e-5}, "max_position": 32768,
+           "layers": [{"type": "attention", "mixer": mixer, "mlp": routed if i % 2 else dense} for i in range(layers)]}
+    start, stop = layers // 4, layers // 4 + max(1, layers // 2)
+    if stop <= layers and layers >= 3:
+        cfg["loop"] = {"start": start, "stop": stop, "times": 2}
+        return cfg, layers + (stop - start)
+    return cfg, layers
+
+
 def llama_config_of(size, layer_runs):
     return {"model_type": "llama", "architectures": ["LlamaForCausalLM"], "num_hidden_layers": layer_runs,
             "hidden_size": size["width"], "num_attention_heads": size["heads"], "num_key_value_heads": size["kv_heads"],
@@ -234,17 +255,17 @@ def llama_config_of(size, layer_runs):
 
 
 def design_run(args):
-    """Prefill and decode throughput of the Menitar design beside Llama at equal sizes (width, heads, head size,
-    feed-forward, vocabulary, as many layers as the other has layer runs), random bfloat16 weights, with the device time
-    of the kernels of a decode step and of a prefill step of each.  Prints one JSON line of its own."""
+    """Prefill and decode throughput of another design (Menitar, Purivik) beside Llama at equal sizes (width, heads, head
+    size, feed-forward, vocabulary, as many layers as the other has layer runs), random bfloat16 weights, with the device
+    time of the kernels of a decode step and of a prefill step of each.  Prints one JSON line of its own."""
     import gc
     import numpy as np
     import torch
     from fllm_amd import Engine, SamplingParams
     size = DESIGN_SIZES[args.design_size]
     layers = args.layers or size["layers"]
-    menitar, layer_runs = menitar_config(size, layers)
-    models = {"menitar": (menitar, size["vocab"]), "llama": (llama_config_of(size, layer_runs), size["vocab"])}
+    design, layer_runs = {"menitar": menitar_config, "purivik": purivik_config}[args.design](size, layers)
+    models = {args.design: (design, size["vocab"]), "llama": (llama_config_of(size, layer_runs), size["vocab"])}
     batches = sorted({1, args.batch, 64})
     steps, warmup = min(args.steps, 96), args.warmup
     held = args.prompt_len + warmup + steps + decode_slack(max(batches), args.prompt_len)
@@ -344,7 +365,7 @@ def main():
     ap.add_argument("--sampled", action="store_true",
                     help="for profiling the sampling kernels: the decode runs draw with temperature 0.8, top-k 50 and top-p 0.9 under a "
                          "repetition penalty of 1.1 and report 5 log-probabilities a token (the headline run is greedy)")
-    ap.add_argument("--design", choices=["menitar"], default=None,
+    ap.add_argument("--design", choices=["menitar", "purivik"], default=None,
                     help="instead of the headline run: prefill and decode of this design beside Llama at equal sizes, with the kernels' "
                          "device times of both; prints a line of its own")
     ap.add_argument("--design-size", choices=sorted(DESIGN_SIZES), default="1.5b", help="with --design: the layer sizes")

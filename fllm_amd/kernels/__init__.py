@@ -89,6 +89,8 @@ def load_library(build_if_missing: bool = True):
         "fllm_experts_gate_up": [c_void, c_int, c_void, c_void, c_int, c_int, c_void, c_int, c_int, c_int, c_void, c_float, c_float,
                                  c_float, c_int, c_void],
         "fllm_experts_down": [c_void, c_void, c_int, c_void, c_int, c_int, c_int, c_void, c_int, c_void],
+        "fllm_experts_grouped": [c_void, c_int, c_void, c_void, c_int, c_int, c_void, c_void, c_int, c_int, c_int, c_int, c_void, c_void,
+                                 c_void, c_float, c_float, c_float, c_void],
         "fllm_attention_sloped": [c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_int,
                                   c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void, c_void],
         "fllm_norm_linear": [c_void, c_void, c_float, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
@@ -150,6 +152,8 @@ def load_library(build_if_missing: bool = True):
     lib.fllm_weight_tiles_elements_gate_up.restype = c_size
     lib.fllm_set_fast_kernels.argtypes = [c_int]
     lib.fllm_set_fast_kernels.restype = None
+    lib.fllm_experts_grouped_work_ints.argtypes = [c_int, c_int]
+    lib.fllm_experts_grouped_work_ints.restype = c_size
     lib.fllm_attention_workspace_bytes.argtypes = [c_int, c_int, c_int, c_int, c_int]
     lib.fllm_attention_workspace_bytes.restype = c_size
     _lib = lib
@@ -844,6 +848,35 @@ class Ops:
         self._check(self.lib.fllm_experts_down(_ptr(act), _ptr(ids), pairs, _ptr(w_down), E, N, inter, _ptr(out),
                                                _DTYPE_CODE[act.dtype], self._stream()))
         return out
+
+    GROUPED_EXPERTS_ROWS = 17      # steps of this many rows and more group their (row, pick) pairs by expert
+
+    def experts_grouped(self, h: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor,
+                        out: torch.Tensor, limit: float = 0.0, alpha: float = 1.0, up_offset: float = 0.0) -> bool:
+        """`experts_gate_up` and `experts_down` in one call on the matrix cores (bfloat16, prompt portions): the pairs are
+        grouped by expert on the device, and an expert multiplies the rows that picked it as tiles.  out float32
+        [rows * top, width].  False: not taken (few rows, float32, sizes that are no multiples of 8), nothing was written."""
+        rows, K = h.shape
+        top = ids.shape[1]
+        if h.dtype != torch.bfloat16 or rows < self.GROUPED_EXPERTS_ROWS or not h.is_cuda:
+            return False
+        E, two_i = w_gate_up.shape[0], w_gate_up.shape[1]
+        N = w_down.shape[1]
+        _need(h.dim() == 2 and h.stride(1) == 1, "h must be a row-major matrix")
+        _dense(w_gate_up, "w_gate_up", h.dtype, (E, two_i, K))
+        _dense(w_down, "w_down", h.dtype, (E, N, two_i // 2))
+        _dense(ids, "ids", torch.int32, (rows, top))
+        _dense(weights, "weights", torch.float32, (rows, top))
+        _dense(out, "out", torch.float32, (rows * top, N))
+        act = torch.empty((rows * top, two_i // 2), dtype=h.dtype, device=h.device)
+        work = torch.empty((int(self.lib.fllm_experts_grouped_work_ints(rows * top, E)),), dtype=torch.int32, device=h.device)
+        code = self.lib.fllm_experts_grouped(_ptr(h), h.stride(0), _ptr(ids), _ptr(weights), rows, top, _ptr(w_gate_up), _ptr(w_down), E,
+                                             two_i // 2, K, N, _ptr(act), _ptr(out), _ptr(work), float(limit), float(alpha),
+                                             float(up_offset), self._stream())
+        if code == 1:
+            return False
+        self._check(code)
+        return True
 
     def _talking_pages(self, k_pages, v_pages, dtype, kv_heads, k_dim, v_dim, page_size, key_chunk):
         _need(key_chunk > 0 and k_dim % key_chunk == 0, f"keys of {k_dim} values cannot lie in chunks of {key_chunk}")

@@ -22,6 +22,7 @@ class PagedAttention(Mixer):
     graph_safe = True      # forward launches kernels only: no per-step decision on the host
     stores_branch = True   # forward(..., branch=t) stores the output projection in t instead of adding it to the stream
     KEY_CHUNK = 8          # values of a key that lie together in a page (csrc/common.h, key_offset)
+    MATRIX_CORE_WIDTHS = (32, 64, 128)      # head sizes the matrix-core attention kernels take
 
     @classmethod
     def tensor_shapes(cls, spec):
@@ -50,6 +51,17 @@ class PagedAttention(Mixer):
             raise ValueError("an attention window must be positive")
         if self.chunk is not None and self.chunk <= 0:
             raise ValueError("a chunk of positions must be positive")
+        # The matrix-core kernels (bfloat16) read keys and values of ONE width of 32, 64 or 128 lanes.  A layer whose two
+        # widths differ, or fit none of the three, runs them all the same: heads are widened to the next such width with
+        # lanes that are zero (zero rows of the q, k and v projections, zero columns of the output projection).  A zero lane
+        # adds exactly nothing to a score or an output, and rotary only touches the first lanes, so the results are the
+        # layer's own; the pages are wider than the layer needs, which is the price (`widen_heads` False: never).
+        self.checkpoint_dims = (self.head_dim, self.v_dim)
+        widest = max(self.head_dim, self.v_dim)
+        fits = next((w for w in self.MATRIX_CORE_WIDTHS if w >= widest), None)
+        if (spec.get("widen_heads", True) and rt.dtype == torch.bfloat16 and fits is not None and hasattr(rt.ops, "tile_for_decode")
+                and (self.head_dim, self.v_dim) != (fits, fits)):
+            self.head_dim = self.v_dim = fits
         # keys lie in chunks of 8 values inside a page where the head size allows it (what the matrix-core kernels read);
         # other head sizes store a head's lanes one by one and run the plain kernels
         self.key_chunk = self.KEY_CHUNK if self.head_dim % self.KEY_CHUNK == 0 else 1
@@ -72,21 +84,34 @@ class PagedAttention(Mixer):
         # (the reference's importer does the same: rust/checkpoint/src/convert.rs:2713-2745).
         self.pairing = 1
         order_q = order_k = None
+        d0, dv0 = self.checkpoint_dims
         if self.position is not None and self.position.pairing == 0:
-            order_q = self._pair_order(self.heads, self.head_dim, self.position.dims).to(rt.device)
-            order_k = self._pair_order(self.kv_heads, self.head_dim, self.position.dims).to(rt.device)
+            order_q = self._pair_order(self.heads, d0, self.position.dims).to(rt.device)
+            order_k = self._pair_order(self.kv_heads, d0, self.position.dims).to(rt.device)
         elif self.position is not None:
             self.pairing = self.position.pairing
         reorder = lambda t, order: t if order is None or t is None else t.index_select(0, order)
+
+        def widen(t, heads, have, want):
+            """Rows of `heads` heads of `have` lanes -> heads of `want` lanes, the new lanes zero."""
+            if t is None or have == want:
+                return t
+            wide = torch.zeros((heads, want) + tuple(t.shape[1:]), dtype=t.dtype, device=t.device)
+            wide[:, :have] = t.view(heads, have, *t.shape[1:])
+            return wide.view(heads * want, *t.shape[1:])
+
         # one matrix for q, k and v: the normed input is read once
-        self.w_qkv = torch.cat([reorder(rt.matrix(weights["q"]), order_q), reorder(rt.matrix(weights["k"]), order_k),
-                                rt.matrix(weights["v"])], dim=0).contiguous()
+        self.w_qkv = torch.cat([widen(reorder(rt.matrix(weights["q"]), order_q), self.heads, d0, self.head_dim),
+                                widen(reorder(rt.matrix(weights["k"]), order_k), self.kv_heads, d0, self.head_dim),
+                                widen(rt.matrix(weights["v"]), self.kv_heads, dv0, self.v_dim)], dim=0).contiguous()
         self.w_o = rt.matrix(weights["o"])
+        if dv0 != self.v_dim:
+            self.w_o = widen(self.w_o.t().contiguous(), self.heads, dv0, self.v_dim).t().contiguous()
         rt.tile_for_decode(self.w_o)
         rt.tile_for_decode(self.w_qkv, priority=1)
-        biases = [reorder(None if weights.get("q_bias") is None else rt.vector(weights["q_bias"]), order_q),
-                  reorder(None if weights.get("k_bias") is None else rt.vector(weights["k_bias"]), order_k),
-                  None if weights.get("v_bias") is None else rt.vector(weights["v_bias"])]
+        biases = [widen(reorder(None if weights.get("q_bias") is None else rt.vector(weights["q_bias"]), order_q), self.heads, d0, self.head_dim),
+                  widen(reorder(None if weights.get("k_bias") is None else rt.vector(weights["k_bias"]), order_k), self.kv_heads, d0, self.head_dim),
+                  widen(None if weights.get("v_bias") is None else rt.vector(weights["v_bias"]), self.kv_heads, dv0, self.v_dim)]
         self.b_qkv = None
         if any(b is not None for b in biases):
             sizes = (self.heads * self.head_dim, self.kv_heads * self.head_dim, self.kv_heads * self.v_dim)

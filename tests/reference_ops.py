@@ -108,13 +108,13 @@ class ReferenceOps:
             if seg < 0:
                 continue
             pos = int(row_pos[r])
-            c, s = cos[pos].double(), sin[pos].double()
+            c, s = (cos[pos].double(), sin[pos].double()) if half else (None, None)
             if pairing == 0:
                 ia, ib = torch.arange(half), torch.arange(half) + half
             else:
                 ia, ib = torch.arange(half) * 2, torch.arange(half) * 2 + 1
             ia, ib = ia.to(qkv.device), ib.to(qkv.device)
-            for h in range(heads + kv_heads):
+            for h in range(heads + kv_heads if half else 0):
                 a, b = view[r, h, ia].double(), view[r, h, ib].double()
                 view[r, h, ia] = (a * c - b * s).to(qkv.dtype)
                 view[r, h, ib] = (b * c + a * s).to(qkv.dtype)

@@ -79,6 +79,28 @@ def test_the_line_of_another_design_beside_its_closest_model():
 
 
 @pytest.mark.gpu
+def test_the_line_of_the_design_with_routed_layers():
+    """`--design purivik`: dense and routed feed-forwards in turn beside Llama at equal sizes."""
+    done = run_bench("--design", "purivik", "--design-size", "small", "--layers", "3", "--steps", "6", "--warmup", "2",
+                     "--repeats", "1")
+    assert done.returncode == 0, done.stderr[-2000:]
+    lines = done.stdout.strip().splitlines()
+    assert len(lines) == 1
+    line = json.loads(lines[0])
+    assert line["layer_runs"] == 4 and line["sizes"]["layers"] == 3 and line["dtype"] == "bf16"
+    for model in ("purivik", "llama"):
+        got = line[model]
+        assert set(got) >= {"decode_b1", "decode_b8", "decode_b64", "prefill", "kernels"}
+        assert got["decode_b64"]["tokens_per_s"] > got["decode_b1"]["tokens_per_s"] > 0
+        assert set(got["kernels"]) == {"prefill_us", "decode_b8_us"}
+    # prompts group the tokens of an expert on the matrix cores and run the matrix-core attention; decode steps fold the
+    # first norm of a layer into its q/k/v product
+    prefill, decode = " ".join(line["purivik"]["kernels"]["prefill_us"]), " ".join(line["purivik"]["kernels"]["decode_b8_us"])
+    assert "grouped_tiles_kernel" in prefill and "attn_tile32_kernel" in prefill and "attention_generic_kernel" not in prefill
+    assert "postnorm_add_kernel" in decode and "attn_decode_kernel" in decode
+
+
+@pytest.mark.gpu
 def test_the_smoke_run_of_the_entry_file():
     """`__graft_entry__.smoke()` in a process of its own, as it is run: a few tokens of a tiny random model on the
     device against the plain implementation."""

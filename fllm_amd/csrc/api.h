@@ -316,12 +316,14 @@ int fllm_experts_gate_up(const void *h, int ldh, const int32_t *ids, const float
 int fllm_experts_down(const void *act, const int32_t *ids, int pairs, const void *w_down, int E, int N, int inter, float *out, int dtype,
                       hipStream_t stream);
 // The same products on the matrix cores (bfloat16): the pairs are grouped by expert on the device and multiplied as tiles of
-// 64 rows.  0: launched; 1: shape declined (the caller runs the plain kernels).  act: scratch, bfloat16 [rows * top, inter];
-// out: float32 [rows * top, N]; work: fllm_experts_grouped_work_ints(rows * top, E) int32 of scratch.
+// 64 or 128 rows.  0: launched; 1: shape declined (the caller runs the plain kernels).  act and xs: scratch, bfloat16
+// [rows * top, inter] and [rows * top, K]; out: float32 [rows * top, N]; work: fllm_experts_grouped_work_ints(rows * top, E)
+// int32 of scratch.
 size_t fllm_experts_grouped_work_ints(int pairs, int E);
+size_t fllm_experts_grouped_plane_floats(int pairs, int E, int N, int inter);   // `planes`: float32 scratch of that many (0: none)
 int fllm_experts_grouped(const void *h, int ldh, const int32_t *ids, const float *weights, int rows, int top, const void *w_gate_up,
-                         const void *w_down, int E, int inter, int K, int N, void *act, float *out, int32_t *work, float limit,
-                         float alpha, float up_offset, hipStream_t stream);
+                         const void *w_down, int E, int inter, int K, int N, void *act, void *xs, float *out, int32_t *work,
+                         float *planes, float limit, float alpha, float up_offset, hipStream_t stream);
 
 #ifdef __cplusplus
 }

@@ -90,7 +90,7 @@ def load_library(build_if_missing: bool = True):
                                  c_float, c_int, c_void],
         "fllm_experts_down": [c_void, c_void, c_int, c_void, c_int, c_int, c_int, c_void, c_int, c_void],
         "fllm_experts_grouped": [c_void, c_int, c_void, c_void, c_int, c_int, c_void, c_void, c_int, c_int, c_int, c_int, c_void, c_void,
-                                 c_void, c_float, c_float, c_float, c_void],
+                                 c_void, c_void, c_void, c_float, c_float, c_float, c_void],
         "fllm_attention_sloped": [c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_void, c_void, c_int, c_void, c_int,
                                   c_int, c_int, c_int, c_int, c_int, c_float, c_int, c_int, c_int, c_void, c_void],
         "fllm_norm_linear": [c_void, c_void, c_float, c_void, c_void, c_void, c_int, c_int, c_int, c_void],
@@ -152,6 +152,8 @@ def load_library(build_if_missing: bool = True):
     lib.fllm_weight_tiles_elements_gate_up.restype = c_size
     lib.fllm_set_fast_kernels.argtypes = [c_int]
     lib.fllm_set_fast_kernels.restype = None
+    lib.fllm_experts_grouped_plane_floats.argtypes = [c_int, c_int, c_int, c_int]
+    lib.fllm_experts_grouped_plane_floats.restype = c_size
     lib.fllm_experts_grouped_work_ints.argtypes = [c_int, c_int]
     lib.fllm_experts_grouped_work_ints.restype = c_size
     lib.fllm_attention_workspace_bytes.argtypes = [c_int, c_int, c_int, c_int, c_int]
@@ -849,7 +851,9 @@ class Ops:
                                                _DTYPE_CODE[act.dtype], self._stream()))
         return out
 
-    GROUPED_EXPERTS_ROWS = 17      # steps of this many rows and more group their (row, pick) pairs by expert
+    GROUPED_EXPERTS_ROWS = 17      # steps of this many rows and more group their (row, pick) pairs by expert,
+    GROUPED_EXPERTS_SHARE = 2      # and smaller ones that have this many pairs an expert: the plain kernels read an expert's
+                                   # matrices once a pair, the grouped ones once a step
 
     def experts_grouped(self, h: torch.Tensor, ids: torch.Tensor, weights: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor,
                         out: torch.Tensor, limit: float = 0.0, alpha: float = 1.0, up_offset: float = 0.0) -> bool:
@@ -858,9 +862,11 @@ class Ops:
         [rows * top, width].  False: not taken (few rows, float32, sizes that are no multiples of 8), nothing was written."""
         rows, K = h.shape
         top = ids.shape[1]
-        if h.dtype != torch.bfloat16 or rows < self.GROUPED_EXPERTS_ROWS or not h.is_cuda:
-            return False
         E, two_i = w_gate_up.shape[0], w_gate_up.shape[1]
+        if h.dtype != torch.bfloat16 or not h.is_cuda:
+            return False
+        if rows < self.GROUPED_EXPERTS_ROWS and rows * top < self.GROUPED_EXPERTS_SHARE * E:
+            return False
         N = w_down.shape[1]
         _need(h.dim() == 2 and h.stride(1) == 1, "h must be a row-major matrix")
         _dense(w_gate_up, "w_gate_up", h.dtype, (E, two_i, K))
@@ -869,9 +875,12 @@ class Ops:
         _dense(weights, "weights", torch.float32, (rows, top))
         _dense(out, "out", torch.float32, (rows * top, N))
         act = torch.empty((rows * top, two_i // 2), dtype=h.dtype, device=h.device)
+        xs = torch.empty((rows * top, K), dtype=h.dtype, device=h.device)      # the rows times their picks' weights
         work = torch.empty((int(self.lib.fllm_experts_grouped_work_ints(rows * top, E)),), dtype=torch.int32, device=h.device)
+        need = int(self.lib.fllm_experts_grouped_plane_floats(rows * top, E, N, two_i // 2))     # a down product cut along K
+        planes = torch.empty((need,), dtype=torch.float32, device=h.device) if need else None
         code = self.lib.fllm_experts_grouped(_ptr(h), h.stride(0), _ptr(ids), _ptr(weights), rows, top, _ptr(w_gate_up), _ptr(w_down), E,
-                                             two_i // 2, K, N, _ptr(act), _ptr(out), _ptr(work), float(limit), float(alpha),
+                                             two_i // 2, K, N, _ptr(act), _ptr(xs), _ptr(out), _ptr(work), _ptr(planes), float(limit), float(alpha),
                                              float(up_offset), self._stream())
         if code == 1:
             return False

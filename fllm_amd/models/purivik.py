@@ -38,7 +38,7 @@ def build_spec(cfg: PurivikConfig) -> ModelSpec:
         mixer = PartSpec(
             "attention",
             {"hidden_size": cfg.width, "num_heads": m.heads, "num_kv_heads": m.kv_heads, "head_dim": m.dim,
-             "value_head_dim": m.vdim, "scale": m.scale, "chunk": m.chunk, "position": position},
+             "value_head_dim": m.vdim, "scale": m.scale, "chunk": m.chunk, "position": position, "widen_heads": True},
             {"q": f"{p}.mix.q", "k": f"{p}.mix.k", "v": f"{p}.mix.v", "o": f"{p}.mix.o"},
         )
         ffn = None

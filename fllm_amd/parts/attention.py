@@ -55,11 +55,12 @@ class PagedAttention(Mixer):
         # widths differ, or fit none of the three, runs them all the same: heads are widened to the next such width with
         # lanes that are zero (zero rows of the q, k and v projections, zero columns of the output projection).  A zero lane
         # adds exactly nothing to a score or an output, and rotary only touches the first lanes, so the results are the
-        # layer's own; the pages are wider than the layer needs, which is the price (`widen_heads` False: never).
+        # layer's own; the pages are wider than the layer needs, which is the price.  An architecture asks for it
+        # with `widen_heads` in the mixer's spec.
         self.checkpoint_dims = (self.head_dim, self.v_dim)
         widest = max(self.head_dim, self.v_dim)
         fits = next((w for w in self.MATRIX_CORE_WIDTHS if w >= widest), None)
-        if (spec.get("widen_heads", True) and rt.dtype == torch.bfloat16 and fits is not None and hasattr(rt.ops, "tile_for_decode")
+        if (spec.get("widen_heads", False) and rt.dtype == torch.bfloat16 and fits is not None and hasattr(rt.ops, "tile_for_decode")
                 and (self.head_dim, self.v_dim) != (fits, fits)):
             self.head_dim = self.v_dim = fits
         # keys lie in chunks of 8 values inside a page where the head size allows it (what the matrix-core kernels read);

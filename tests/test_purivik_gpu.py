@@ -173,8 +173,10 @@ def test_experts_grouped_on_the_matrix_cores(ops, ref, rows, width, inter, exper
     keep = torch.randperm(rows, generator=g)[:max(17, rows // 3)].sort()[0]
     part = torch.empty(len(keep) * top, width, dtype=torch.float32, device=DEV)
     assert ops.experts_grouped(h[keep].to(DEV), ids[keep].to(DEV), weights[keep].to(DEV), w_gate_up.to(DEV), w_down.to(DEV), part, limit, alpha, offset)
-    assert torch.equal(part.view(len(keep), top, width), out.view(rows, top, width)[keep.to(DEV)])
-    assert not ops.experts_grouped(h[:4].to(DEV), ids[:4].to(DEV), weights[:4].to(DEV), w_gate_up.to(DEV), w_down.to(DEV), part[:4 * top])
+    # (to the last bits only: few rows cut the down product along K, and the slices are summed in another order)
+    close(part.view(len(keep), top, width), out.view(rows, top, width)[keep.to(DEV)].double(), 1e-5, 1e-5 * want.abs().max().item(), "other company")
+    few = 1 if top > 1 else 2           # fewer than two pairs an expert: left to the plain kernels
+    assert not ops.experts_grouped(h[:few].to(DEV), ids[:few].to(DEV), weights[:few].to(DEV), w_gate_up.to(DEV), w_down.to(DEV), part[:few * top])
 
 
 # ---------------------------------------------------------------------------------------------

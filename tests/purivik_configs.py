@@ -61,8 +61,17 @@ D = config(128, 160, [layer(8, 2, 64, 64, chunk=80, rot=(32, 25000.0), scaling=(
 E = config(68, 77, [layer(3, 1, 24, 40, chunk=7, rot=(10, 77.0), scaling=(2.5, 0.5, 3.0, 30), mlp=("moe", 18, 7, 2), scale=0.3),
                     layer(3, 1, 24, 40, chunk=7, rot=(10, 77.0), mlp=("dense", 50, 0.9), scale=0.3)], loop=(0, 2, 2), embedding_scale=2.0,
            residual_mult=0.8)
-CONFIGS = {"A": A, "B": B, "C": C, "D": D, "E": E}
-PAGE_SIZES = {"A": 8, "B": 16, "C": 8, "D": 16, "E": 16}
+# F: heads wider than any matrix-core kernel takes (keys of 160 lanes, values of 136: the plain attention in both precisions),
+# a single expert (always picked, its score still scales its input), the first layer looped
+F = config(96, 100, [layer(4, 2, 160, 136, chunk=50, rot=(40, 1000000.0), scaling=(8.0, 1.0, 4.0, 128), mlp=("moe", 32, 1, 1)),
+                     layer(4, 2, 160, 136, chunk=50, rot=(40, 1000000.0), scaling=(8.0, 1.0, 4.0, 128), mlp=("dense", 72, 1.5))],
+           loop=(0, 1, 2), residual_mult=0.7)
+# G: keys of 80 and values of 96 lanes (widened to 128 in bfloat16), chunks of 150 positions (no multiple of a page or of a
+# key tile) under requests of several hundred tokens, one pick of six experts
+G = config(128, 200, [layer(8, 4, 80, 96, chunk=150, rot=(20, 50000.0), mlp=("moe", 40, 6, 1)),
+                      layer(8, 4, 80, 96, chunk=150, rot=(20, 50000.0), mlp=("dense", 160, 1.0))], embedding_scale=6.0, residual_mult=0.7)
+CONFIGS = {"A": A, "B": B, "C": C, "D": D, "E": E, "F": F, "G": G}
+PAGE_SIZES = {"A": 8, "B": 16, "C": 8, "D": 16, "E": 16, "F": 16, "G": 16}
 
 
 def bf16_round(a):

@@ -150,7 +150,8 @@ def test_the_loader_names_what_does_not_fit():
 
 
 # ---- the engine's logic -------------------------------------------------------------------------------------------------
-@pytest.mark.parametrize("name,lengths", [("A", [5, 30, 61]), ("B", [45, 83]), ("C", [9, 50]), ("D", [100, 37]), ("E", [20, 51])])
+@pytest.mark.parametrize("name,lengths", [("A", [5, 30, 61]), ("B", [45, 83]), ("C", [9, 50]), ("D", [100, 37]), ("E", [20, 51]),
+                                          ("F", [60, 23]), ("G", [170, 40])])
 @pytest.mark.parametrize("family", ["whole", "last", "portions", "mixed"])
 def test_every_way_of_cutting_gives_the_plain_logits(tmp_path, name, lengths, family):
     vocab = pc.CONFIGS[name]["vocab"]

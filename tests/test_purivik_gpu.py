@@ -359,7 +359,8 @@ def test_the_matrix_core_attention_takes_chunks_of_positions(ops):
 # ---------------------------------------------------------------------------------------------
 # the engine
 # ---------------------------------------------------------------------------------------------
-LENGTHS = {"A": [5, 30, 61, 100, 49], "B": [45, 83, 161, 2, 120], "C": [9, 50, 300, 130], "D": [100, 37, 250, 81, 160], "E": [31, 2, 75, 120]}
+LENGTHS = {"A": [5, 30, 61, 100, 49], "B": [45, 83, 161, 2, 120], "C": [9, 50, 300, 130], "D": [100, 37, 250, 81, 160], "E": [31, 2, 75, 120], "F": [60, 130, 17],
+           "G": [700, 333, 64, 461]}
 # about three times the largest error any case here has shown on the MI355X (float32 5.3e-6, bfloat16 2.5e-2).  The float32
 # figure is that of the configurations which rotate every lane of a head: the angles are float32 products of a position and
 # a frequency, as the design has them, and at positions beyond 100 they differ from the plain implementation's float64
@@ -401,7 +402,7 @@ def check(got, plain, dtype, what):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D", "E", "F", "G"])
 @pytest.mark.parametrize("family", ["whole", "last40", "portions", "mixed"])
 def test_replay(models, tmp_path, name, dtype, family):
     folder, cfg, requests, plain, _ = models[name, dtype]

@@ -27,6 +27,26 @@ __device__ __forceinline__ float lane_dot8(const float *__restrict__ xs, const b
     }
     return acc;
 }
+// R weight rows against the same x at once, 8 neighbours a load and row: the loads of all rows are in flight together, which
+// is what a workgroup that streams a few rows of a matrix is short of.  Row r's sum is added in the order lane_dot8 adds it.
+template <int R>
+__device__ __forceinline__ void lane_dots8(const float *__restrict__ xs, const bf16_t *const (&w)[R], int K, int lane, float (&acc)[R]) {
+#pragma unroll
+    for (int r = 0; r < R; r++) acc[r] = 0.f;
+    for (int c = lane * 8; c < K; c += kWave * 8) {
+        bf16x8_t w8[R];
+#pragma unroll
+        for (int r = 0; r < R; r++) w8[r] = __builtin_nontemporal_load((const bf16x8_t *)(w[r] + c));
+        float x8[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) x8[e] = xs[c + e];
+#pragma unroll
+        for (int r = 0; r < R; r++)
+#pragma unroll
+            for (int e = 0; e < 8; e++) acc[r] = fmaf(x8[e], (float)w8[r][e], acc[r]);
+    }
+}
+
 template <typename T> __device__ __forceinline__ float row_dot(const float *xs, const T *w, int K, int lane, bool vec);
 template <> __device__ __forceinline__ float row_dot<float>(const float *xs, const float *w, int K, int lane, bool) {
     return wave_sum(lane_dot<float>(xs, w, K, lane));
@@ -107,6 +127,39 @@ expert_rows_kernel(const T *__restrict__ x, int ldx, const int32_t *__restrict__
     }
     __syncthreads();
     const bool vec = sizeof(T) == 2 && K % 8 == 0 && ((uintptr_t)w & 15) == 0;
+    if constexpr (sizeof(T) == 2) {
+        // bfloat16 rows of whole 16-byte pieces: the wave's columns at once (their sums are those of the loop below, bit for bit)
+        const int c0 = blockIdx.x * kCols + wave * kColsPerWave;
+        if (vec && c0 + kColsPerWave <= N) {
+            if (MODE == 0) {
+                const bf16_t *base = (const bf16_t *)w + ((size_t)e * 2 * N + c0) * K;
+                const bf16_t *const rows[4] = {base, base + K, base + (size_t)N * K, base + (size_t)N * K + K};
+                float acc[4];
+                lane_dots8<4>(xs, rows, K, lane, acc);
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    float g = wave_sum(acc[j]), u = wave_sum(acc[2 + j]);
+                    if (limit > 0.f) {
+                        g = fminf(g, limit);
+                        u = fminf(fmaxf(u, -limit), limit);
+                    }
+                    if (lane == 0) act[pair * N + c0 + j] = from_f32<T>(g / (1.0f + expf(-alpha * g)) * (u + up_offset));
+                }
+            } else {
+                const bf16_t *base = (const bf16_t *)w + ((size_t)e * N + c0) * K;
+                const bf16_t *const rows[2] = {base, base + K};
+                float acc[2];
+                lane_dots8<2>(xs, rows, K, lane, acc);
+#pragma unroll
+                for (int j = 0; j < 2; j++) {
+                    const float y = wave_sum(acc[j]);
+                    if (lane == 0) out[pair * N + c0 + j] = y;
+                }
+            }
+            return;
+        }
+    }
+    static_assert(kColsPerWave == 2, "the wave's columns at once are two");
 #pragma unroll
     for (int j = 0; j < kColsPerWave; j++) {
         const int c = blockIdx.x * kCols + wave * kColsPerWave + j;

@@ -462,7 +462,7 @@ def test_first_tokens_and_long_decoding(models, tmp_path, name, dtype):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("name", ["A", "D"])
+@pytest.mark.parametrize("name", ["A", "C", "D"])      # C: two decode rows are six pairs over three experts, grouped inside the graph
 def test_decode_graphs_and_eager_steps_agree(models, tmp_path, name, dtype):
     folder, cfg, requests, plain, _ = models[name, dtype]
     steps = tt.number(tt.last_tokens_one_by_one(requests) + tt.mixed(requests, seed=21, decode_tail=40))

@@ -55,8 +55,8 @@ template <> __device__ __forceinline__ float row_dot<bf16_t>(const float *xs, co
     return wave_sum(vec ? lane_dot8(xs, w, K, lane) : lane_dot<bf16_t>(xs, w, K, lane));
 }
 
-// Router: z = W h in float32, score = sigmoid(z) (mode 0) ; the `top` largest scores of a row, ties to the lower index;
-// weights[r, k] = the score of pick k (mode 0) .  One workgroup a row; scores through LDS.
+// Router: z = W h in float32, score = sigmoid(z); the `top` largest scores of a row, ties to the lower index;
+// weights[r, k] = the score of pick k.  One workgroup a row; scores through LDS.
 template <typename T>
 __global__ void __launch_bounds__(kBlock)
 route_kernel(const T *__restrict__ h, int ldh, const T *__restrict__ w, int K, int E, int top, int32_t *__restrict__ ids,

@@ -28,6 +28,12 @@ Roles and their interfaces:
                 number of tokens the request held before this step; so the state a mixer finds is the one it left after
                 position seg_pos_start[s] - 1.
   feed_forward  forward(ctx, h[R,H], residual_f32[R,H]) adds its output to `residual`.
+                A stored branch (optional, mixers and feed-forwards): a part with `stores_branch = True` also takes
+                `branch=t` (float32) and then STORES its output in t instead of adding it to `residual` (which may be
+                None), for arrangements that treat a part's output before it joins the stream (a norm behind the part).
+                t has `branch_parts` rows a token (1 unless the part says otherwise: a token's experts leave their
+                outputs one after the other, and whoever adds the branch sums them in that order).  An arrangement hands
+                a part without the attribute a zeroed stand-in for the stream, so every part fits.
   block         forward(ctx, residual_f32[R,H], binding) runs norms, mixer and feed-forward.  It is built with
                 mixer=, feed_forward= (None for a layer without one), norms= (by the names the layer's spec
                 uses) and, only when the spec lists any, extras= (further parts by name).  A block

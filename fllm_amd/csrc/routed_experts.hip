@@ -89,6 +89,7 @@ route_kernel(const T *__restrict__ h, int ldh, const T *__restrict__ w, int K, i
             const int other_at = __shfl_xor(at, o, kWave);
             if (other > best || (other == best && other_at < at)) best = other, at = other_at;
         }
+        if (at < 0 || at >= E) at = k;           // scores that compare with nothing (NaN rows): still an expert of the stack
         if (lane == 0) {
             ids[r * top + k] = at;
             weights[r * top + k] = best;
